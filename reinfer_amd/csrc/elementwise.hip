@@ -1,0 +1,245 @@
+// Row kernels of the step: embedding rows, fused residual-add + RMSNorm,
+// fused per-head q/k norm + rotation + cache write, SiLU gate.
+// Sums of squares, rsqrt, rotation angles and the residual sum are float;
+// one rounding at the store.
+#include "common.h"
+#include "reinfer_hip.h"
+
+thread_local char ra_error_text[512] = {0};
+
+int ra_fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(ra_error_text, sizeof(ra_error_text), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+extern "C" const char* ra_last_error(void) { return ra_error_text; }
+extern "C" int ra_abi_version(void) { return RA_ABI_VERSION; }
+
+// ---------------------------------------------------------------------------
+// embedding rows into the float residual stream: out[t, :] = table[ids[t], :]
+// (reference: gather_row, crates/cuda/kernels/dense_kernels.cu:329-336)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int h) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * h;
+  float* o = out + (size_t)t * h;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = to_f32(row[i]);
+}
+
+extern "C" int ra_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens,
+                        int hidden, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && hidden > 0, "embed: empty input (%d tokens, width %d)", n_tokens, hidden);
+  if (table_dtype == RA_F32)
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, out, hidden);
+  else if (table_dtype == RA_BF16)
+    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden);
+  else
+    return ra_fail("embed: unknown dtype tag %d", table_dtype);
+  RA_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Fused residual add + RMSNorm (any width).
+//   in place (rows == null):  resid[r] += delta[r];  out[r] = rms(resid[r]) * w
+//   gathered (rows != null):  out[i] = rms(resid[rows[i]] + delta[rows[i]]) * w
+// y = x * rsqrt(mean(x^2) + eps) * w   (crates/cuda/kernels/dense_kernels.cu:59-88,
+// fused add form :257-274; there limited to n <= 1024 and one row).
+// ---------------------------------------------------------------------------
+template <typename TA, typename TW>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
+                                   const TW* __restrict__ w, TA* __restrict__ out,
+                                   const int* __restrict__ rows, int h, float eps) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * h;
+  const TA* dl = delta ? delta + src * h : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    float v = x[i];
+    if (dl) {
+      v += to_f32(dl[i]);
+      if (!rows) x[i] = v;      // the same thread reads it back below
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss / (float)h + eps);
+  TA* o = out + (size_t)r * h;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    float v = x[i];
+    if (dl && rows) v += to_f32(dl[i]);
+    o[i] = from_f32<TA>(v * rstd * to_f32(w[i]));
+  }
+}
+
+extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype,
+                              void* out, int act_dtype, const int* rows, int n_rows, int hidden,
+                              float eps, hipStream_t stream) {
+  RA_CHECK(n_rows > 0 && hidden > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_rows, hidden);
+  const int threads = hidden >= 2048 ? 512 : 256;
+#define RA_GO(TA, TW)                                                                           \
+  add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta,          \
+                                                             (const TW*)weight, (TA*)out, rows, \
+                                                             hidden, eps)
+  if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GO(float, float);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GO(bf16_t, bf16_t);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GO(bf16_t, float);
+  else return ra_fail("add_rmsnorm: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
+#undef RA_GO
+  RA_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Fused per-head RMSNorm of q and k, rotation, and cache write.
+// qkv: [T, (Hq + 2 Hkv) * d]; q heads are normalised + rotated in place, k heads
+// are normalised + rotated and stored at the token's cache slot, v heads are
+// copied there. One wavefront per (token, head).
+//   head norm: u * rsqrt(mean(u^2) + eps) * g, one g[d] for all heads, before the
+//     rotation (crates/cuda/kernels/dense_kernels.cu:92-123; engine.rs:4122-4147)
+//   rotation: pairs (j, j + R/2) [style 0, half split] or (2j, 2j+1) [style 1],
+//     angle = pos * inv_freq[j] (dense_kernels.cu:125-139)
+//   cache: [block][kv head][slot in block][d]  (write: dense_kernels.cu:298-318)
+// ---------------------------------------------------------------------------
+#define QK_WAVES 4
+#define QK_MAX_D 512
+
+template <typename TA, typename TW>
+__global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w,
+                                          const TW* __restrict__ k_w, float eps,
+                                          const int* __restrict__ positions,
+                                          const float* __restrict__ inv_freq, int rotary_dim,
+                                          int rope_style, const int* __restrict__ slots,
+                                          TA* __restrict__ kcache, TA* __restrict__ vcache,
+                                          int block_size, int Hq, int Hkv, int d) {
+  __shared__ float buf[QK_WAVES][QK_MAX_D];
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = threadIdx.x / RA_WAVE;
+  const int t = blockIdx.y;
+  const int head = blockIdx.x * QK_WAVES + wave;
+  const int n_heads = Hq + 2 * Hkv;
+  const bool live = head < n_heads;
+  TA* u = qkv + ((size_t)t * n_heads + (live ? head : 0)) * d;
+  const bool is_q = head < Hq;
+  const bool is_k = !is_q && head < Hq + Hkv;
+  const int kvh = is_q ? 0 : (is_k ? head - Hq : head - Hq - Hkv);
+  const int slot = slots[t];
+  TA* dst = nullptr;            // where a k or v head goes
+  if (live && !is_q && slot >= 0) {
+    const size_t blk = (size_t)(slot / block_size);
+    const int off = slot % block_size;
+    dst = (is_k ? kcache : vcache) + ((blk * Hkv + kvh) * block_size + off) * d;
+  }
+  float* b = buf[wave];
+  float ss = 0.f;
+  if (live) {
+    for (int i = lane; i < d; i += RA_WAVE) {
+      float v = to_f32(u[i]);
+      b[i] = v;
+      ss += v * v;
+    }
+  }
+  __syncthreads();
+  if (!live) return;
+  if (!is_q && !is_k) {          // v head: plain copy
+    if (dst)
+      for (int i = lane; i < d; i += RA_WAVE) dst[i] = from_f32<TA>(b[i]);
+    return;
+  }
+  const TW* w = is_q ? q_w : k_w;
+  float rstd = 1.f;
+  if (w) {
+    ss = wave_sum(ss);
+    rstd = rsqrtf(ss / (float)d + eps);
+  }
+  TA* o = is_q ? u : dst;
+  if (!o) return;
+  const float pos = (float)positions[t];
+  const int half = rotary_dim / 2;
+  for (int j = lane; j < half; j += RA_WAVE) {
+    const int i0 = rope_style == 0 ? j : 2 * j;
+    const int i1 = rope_style == 0 ? j + half : 2 * j + 1;
+    float a = b[i0] * rstd, c = b[i1] * rstd;
+    if (w) {
+      a *= to_f32(w[i0]);
+      c *= to_f32(w[i1]);
+    }
+    float sn, cs;
+    sincosf(pos * inv_freq[j], &sn, &cs);
+    o[i0] = from_f32<TA>(a * cs - c * sn);
+    o[i1] = from_f32<TA>(a * sn + c * cs);
+  }
+  for (int i = rotary_dim + lane; i < d; i += RA_WAVE) {
+    float a = b[i] * rstd;
+    if (w) a *= to_f32(w[i]);
+    o[i] = from_f32<TA>(a);
+  }
+}
+
+extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
+                                     int weight_dtype, float eps, const int* positions,
+                                     const float* inv_freq, int rotary_dim, int rope_style,
+                                     const int* slots, void* kcache, void* vcache, int block_size,
+                                     int n_tokens, int Hq, int Hkv, int d, hipStream_t stream) {
+  RA_CHECK(n_tokens > 0, "qk_norm_rope_cache: no tokens");
+  RA_CHECK(Hq > 0 && Hkv > 0 && d > 0, "qk_norm_rope_cache: bad head sizes (%d, %d, %d)", Hq, Hkv, d);
+  RA_CHECK(d <= QK_MAX_D, "qk_norm_rope_cache: head size %d above the supported %d", d, QK_MAX_D);
+  RA_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0,
+           "qk_norm_rope_cache: rotary width %d must be even and <= head size %d", rotary_dim, d);
+  RA_CHECK(rope_style == 0 || rope_style == 1, "qk_norm_rope_cache: unknown rotation style %d", rope_style);
+  RA_CHECK((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_rope_cache: q and k norm weights go together");
+  RA_CHECK(block_size > 0, "qk_norm_rope_cache: block size %d", block_size);
+  RA_CHECK(n_tokens <= 65535, "qk_norm_rope_cache: %d tokens in one launch (max 65535)", n_tokens);
+  dim3 grid((Hq + 2 * Hkv + QK_WAVES - 1) / QK_WAVES, n_tokens);
+#define RA_GO(TA, TW)                                                                              \
+  qk_norm_rope_cache_kernel<TA, TW><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(                      \
+      (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, rotary_dim,   \
+      rope_style, slots, (TA*)kcache, (TA*)vcache, block_size, Hq, Hkv, d)
+  if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GO(float, float);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GO(bf16_t, bf16_t);
+  else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GO(bf16_t, float);
+  else return ra_fail("qk_norm_rope_cache: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
+#undef RA_GO
+  RA_LAUNCH_CHECK("qk_norm_rope_cache");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// SiLU gate: out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g / (1 + exp(-g))
+// (crates/cuda/kernels/dense_kernels.cu:202-213)
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = to_f32(gu[t * 2 * I + i]);
+    const float u = to_f32(gu[t * 2 * I + I + i]);
+    out[idx] = from_f32<TA>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
+                           hipStream_t stream) {
+  RA_CHECK(n_tokens > 0 && intermediate > 0, "silu_mul: empty input");
+  const size_t total = (size_t)n_tokens * intermediate;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535 * 4) blocks = 65535 * 4;
+  if (act_dtype == RA_F32)
+    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, total);
+  else if (act_dtype == RA_BF16)
+    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, total);
+  else
+    return ra_fail("silu_mul: unknown dtype tag %d", act_dtype);
+  RA_LAUNCH_CHECK("silu_mul");
+  return 0;
+}

@@ -1,0 +1,46 @@
+// C interface of the gfx950 kernel library. Every entry point checks its
+// arguments on the host, launches on the given stream and returns 0, or
+// returns non-zero with a message in ra_last_error(). Pointers are device
+// memory unless said otherwise. dtype tags: 0 = float, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#define RA_ABI_VERSION 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ra_last_error(void);
+int ra_abi_version(void);
+
+int ra_embed(const void* table, int table_dtype, const int* ids, float* out, int n_tokens, int hidden,
+             hipStream_t stream);
+
+int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype, void* out,
+                   int act_dtype, const int* rows, int n_rows, int hidden, float eps, hipStream_t stream);
+
+int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
+                          int weight_dtype, float eps, const int* positions, const float* inv_freq,
+                          int rotary_dim, int rope_style, const int* slots, void* kcache, void* vcache,
+                          int block_size, int n_tokens, int Hq, int Hkv, int d, hipStream_t stream);
+
+int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
+                hipStream_t stream);
+
+int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                       const void* vcache, int act_dtype, const int* block_tables, int max_blocks,
+                       const int* seq_of_token, const int* positions, int n_tokens, int block_size,
+                       int Hq, int Hkv, int d, float scale, int window, hipStream_t stream);
+
+int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int in_dtype, int out_dtype,
+                  int M, int N, int K, int lda, int ldc, hipStream_t stream);
+
+int ra_sample_slices(int vocab);
+int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,
+              const long long* seeds, const int* positions, float* scratch_val, int* scratch_idx,
+              int* tokens, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

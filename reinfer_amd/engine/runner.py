@@ -1,0 +1,210 @@
+"""The step function: model + cache on one GPU.
+
+``ModelRunner.step(entries)`` runs exactly the tokens it is given, as one
+batch, from the cache that earlier steps left, and returns float32 logits at
+the wanted places. Generation (scheduler + sampler) and trace replay both call
+this one function; neither has a forward pass of its own.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheGroupSpec, CacheManager, OutOfBlocks, plan_groups
+from ..config import load_config
+from ..config.schema import ModelSpec
+from ..models import DecoderModel, declare_params
+from ..parts import KVNeed, LayerCache, StateNeed
+from ..weights import check_tensors, load_weights, random_tensors, storage_dtype
+from .batch import StepBatch, StepEntry, build_step_batch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+           "fp32": torch.float32, "f32": torch.float32}
+
+
+class StepError(ValueError):
+    """A step was asked for something it cannot run (checked before any launch);
+    the reference's step checks the same on the host (crates/cuda/src/engine.rs:5854-5943)."""
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype {dtype}: the engine runs in bfloat16 or float32")
+        return dtype
+    try:
+        return _DTYPES[str(dtype)]
+    except KeyError:
+        raise ValueError(f"dtype {dtype!r}: expected bfloat16 or float32") from None
+
+
+class ModelRunner:
+    def __init__(self, spec: ModelSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
+                 device: torch.device, *, block_size: int = 16, num_blocks: Optional[int] = None,
+                 max_tokens: Optional[int] = None, max_seqs: int = 64,
+                 max_model_len: Optional[int] = None, memory_fraction: float = 0.9):
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+        self.block_size = int(block_size)
+        self.max_model_len = min(max_model_len or spec.max_positions, spec.max_positions)
+        self.model = DecoderModel(spec, weights, dtype, device)
+        needs = self.model.cache_needs()
+
+        # which run-order entries keep keys of their own, and with which window
+        windows: List[Optional[int]] = []
+        for e, need in zip(spec.run_order, needs):
+            if isinstance(need, KVNeed) and e.cache_from is None:
+                windows.append(need.window)
+            else:
+                windows.append(None)
+        groups = plan_groups(windows)
+        if not groups:
+            groups = [CacheGroupSpec(window=0, entries=())]     # block tables exist even if unused
+        self.groups = groups
+        group_of = {i: g for g, gs in enumerate(groups) for i in gs.entries}
+
+        if num_blocks is None:
+            if max_tokens is not None:
+                num_blocks = max(1, -(-int(max_tokens) // self.block_size))
+            else:
+                num_blocks = self._blocks_that_fit(needs, windows, memory_fraction)
+        self.num_blocks = int(num_blocks)
+        self.manager = CacheManager(groups, self.block_size, [self.num_blocks] * len(groups), max_seqs)
+
+        # device side of the cache
+        self.caches: List[Optional[LayerCache]] = []
+        for i, (e, need) in enumerate(zip(spec.run_order, needs)):
+            if isinstance(need, KVNeed):
+                if e.cache_from is None:
+                    shape = (self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
+                    k = torch.zeros(shape, dtype=dtype, device=device)
+                    v = torch.zeros(shape, dtype=dtype, device=device)
+                    self.caches.append(LayerCache(k=k, v=v, group=group_of[i], writes=True))
+                else:
+                    src = self.caches[e.cache_from]
+                    src_need = needs[e.cache_from]
+                    if not isinstance(src_need, KVNeed) or (src_need.num_kv_heads, src_need.head_dim) != \
+                            (need.num_kv_heads, need.head_dim):
+                        raise ValueError(f"run entry {i} cannot read the cache of entry {e.cache_from}: "
+                                         "different heads")
+                    self.caches.append(LayerCache(k=src.k, v=src.v, group=src.group, writes=False))
+            elif isinstance(need, StateNeed):
+                state = torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device)
+                self.caches.append(LayerCache(state=state))
+            else:
+                self.caches.append(None)
+
+    # ------------------------------------------------------------ building
+    @classmethod
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **limits) -> "ModelRunner":
+        cfg = load_config(model_dir)
+        spec = cfg.to_spec()
+        tdtype = parse_dtype(dtype)
+        dev = torch.device(device)
+        weights = load_weights(model_dir, declare_params(spec), tdtype, dev)
+        return cls(spec, weights, tdtype, dev, **limits)
+
+    @classmethod
+    def from_config(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0",
+                    weights: Optional[Dict[str, torch.Tensor]] = None, **limits) -> "ModelRunner":
+        """Random weights drawn on ``device`` (or the tensors given), no folder."""
+        spec = config.to_spec()
+        tdtype = parse_dtype(dtype)
+        dev = torch.device(device)
+        decls = declare_params(spec)
+        if weights is None:
+            weights = random_tensors(decls, seed, tdtype, dev)
+        else:
+            check_tensors("weights", decls, weights)
+            by = {d.name: d for d in decls}
+            weights = {n: t.to(storage_dtype(by[n], t.dtype, tdtype)).to(dev) for n, t in weights.items()}
+        return cls(spec, weights, tdtype, dev, **limits)
+
+    def _blocks_that_fit(self, needs, windows, fraction: float) -> int:
+        """Blocks per group from free device memory: the reference's budget,
+        capacity = utilisation * total - weights, pages = capacity / page bytes
+        (crates/memory/src/budget.rs:99-117)."""
+        per_block = 0
+        size = torch.empty((), dtype=self.dtype).element_size()
+        for need, w in zip(needs, windows):
+            if w is not None:
+                per_block += 2 * need.num_kv_heads * self.block_size * need.head_dim * size
+        if per_block == 0:
+            return 1
+        if self.device.type != "cuda":
+            return 256
+        free, total = torch.cuda.mem_get_info(self.device)
+        usable = free - (1.0 - fraction) * total
+        blocks = int(usable // per_block)
+        # no request can hold more than max_model_len tokens; 64 requests is the cap on live ones
+        cap = 64 * (-(-self.max_model_len // self.block_size))
+        return max(1, min(blocks, cap))
+
+    # ----------------------------------------------------------- requests
+    def add_request(self, rid: Hashable) -> None:
+        self.manager.add(rid)
+
+    def free_request(self, rid: Hashable) -> None:
+        self.manager.free(rid)
+
+    def has_request(self, rid: Hashable) -> bool:
+        return rid in self.manager
+
+    def num_tokens(self, rid: Hashable) -> int:
+        return self.manager.get(rid).num_tokens
+
+    # --------------------------------------------------------------- step
+    def check_entries(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one request")
+        seen = set()
+        V = self.spec.vocab_size
+        for e in entries:
+            if e.rid in seen:
+                raise StepError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+            if e.rid not in self.manager:
+                raise StepError(f"request {e.rid!r} is not live")
+            if len(e.tokens) == 0:
+                raise StepError(f"request {e.rid!r} brings no tokens")
+            for tok in e.tokens:
+                if not 0 <= int(tok) < V:
+                    raise StepError(f"request {e.rid!r}: token {tok} outside the vocabulary of {V}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise StepError(f"request {e.rid!r}: logits wanted at {w} of {len(e.tokens)} tokens")
+            total = self.manager.get(e.rid).num_tokens + len(e.tokens)
+            if total > self.max_model_len:
+                raise StepError(f"request {e.rid!r}: {total} tokens exceed the context of {self.max_model_len}")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries' tokens as one batch; logits [wanted, vocab] float32,
+        in the order of the entries and of each entry's ``want``."""
+        self.check_entries(entries)
+        growth = [(e.rid, self.manager.get(e.rid).num_tokens + len(e.tokens)) for e in entries]
+        if not self.manager.can_grow(growth):
+            need = [sum(self.manager.blocks_needed(r, t)[g] for r, t in growth)
+                    for g in range(len(self.groups))]
+            g = max(range(len(self.groups)), key=lambda i: need[i] - self.manager.pools[i].num_free)
+            raise OutOfBlocks(g, need[g], self.manager.pools[g].num_free)
+        for rid, total in growth:
+            self.manager.grow(rid, total)
+        batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
+        logits = self.forward(batch)
+        for rid, total in growth:
+            self.manager.commit(rid, total)
+        return logits
+
+    def forward(self, batch: StepBatch) -> torch.Tensor:
+        with torch.no_grad():
+            if batch.num_logit_rows == 0:
+                # still run the layers: the step's keys and values must be stored
+                self._forward_no_logits(batch)
+                return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+            return self.model.forward(batch, self.caches)
+
+    def _forward_no_logits(self, batch: StepBatch) -> None:
+        self.model.forward_layers(batch, self.caches)

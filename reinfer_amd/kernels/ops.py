@@ -1,0 +1,205 @@
+"""Tensor-level entry points of the kernel library.
+
+Each function checks on the host that shapes, dtypes, devices and strides are
+what the kernel assumes, and only then launches on torch's current stream. The
+parts call these through :func:`reinfer_amd.kernels.current`.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import library
+
+_TAG = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _tag(t: torch.Tensor, what: str) -> int:
+    try:
+        return _TAG[t.dtype]
+    except KeyError:
+        raise TypeError(f"{what}: dtype {t.dtype} is not float32 or bfloat16") from None
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise library.KernelLibraryError(
+                "the kernels run on the GPU only: got a tensor on " + str(t.device))
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _int32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise TypeError(f"{what}: expected a contiguous int32 tensor, got {t.dtype}")
+    if n is not None and t.numel() < n:
+        raise ValueError(f"{what}: {t.numel()} entries, need {n}")
+
+
+class HipKernels:
+    """The product's kernels. Stateless apart from the loaded library."""
+
+    name = "hip-gfx950"
+
+    def __init__(self):
+        library.load()
+
+    # ------------------------------------------------------------------ rows
+    def embed(self, table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+        _dev(table, ids, out)
+        T, h = out.shape
+        if table.dim() != 2 or table.shape[1] != h or not table.is_contiguous():
+            raise ValueError(f"embed: table {tuple(table.shape)} does not have rows of width {h}")
+        if out.dtype != torch.float32 or not out.is_contiguous():
+            raise TypeError("embed: the residual stream is contiguous float32")
+        _int32(ids, "embed ids", T)
+        library.call("ra_embed", table.data_ptr(), _tag(table, "embed table"), ids.data_ptr(),
+                     out.data_ptr(), T, h, _stream())
+
+    def add_rmsnorm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                    eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+        _dev(resid, delta, weight, out, rows)
+        h = resid.shape[-1]
+        n = out.shape[0]
+        if resid.dtype != torch.float32 or not resid.is_contiguous():
+            raise TypeError("add_rmsnorm: the residual stream is contiguous float32")
+        if weight.shape != (h,) or out.shape[-1] != h or not out.is_contiguous():
+            raise ValueError(f"add_rmsnorm: width {h}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        if delta is not None:
+            if delta.shape != resid.shape or delta.dtype != out.dtype or not delta.is_contiguous():
+                raise ValueError("add_rmsnorm: delta must match the residual's shape and the output's dtype")
+        if rows is None:
+            if n != resid.shape[0]:
+                raise ValueError("add_rmsnorm: in-place form needs one output row per residual row")
+        else:
+            _int32(rows, "add_rmsnorm rows", n)
+        library.call("ra_add_rmsnorm", resid.data_ptr(), _ptr(delta), weight.data_ptr(),
+                     _tag(weight, "norm weight"), out.data_ptr(), _tag(out, "add_rmsnorm out"),
+                     _ptr(rows), n, h, float(eps), _stream())
+
+    def qk_norm_rope_cache(self, qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
+                           k_weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
+                           inv_freq: torch.Tensor, rotary_dim: int, rope_style: int,
+                           slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                           num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+        _dev(qkv, q_weight, k_weight, positions, inv_freq, slots, kcache, vcache)
+        T = qkv.shape[0]
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        if qkv.shape != (T, width) or not qkv.is_contiguous():
+            raise ValueError(f"qk_norm_rope_cache: qkv {tuple(qkv.shape)}, expected [T, {width}] contiguous")
+        if kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[1] != num_kv_heads \
+                or kcache.shape[3] != head_dim or not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise ValueError(f"qk_norm_rope_cache: cache {tuple(kcache.shape)} is not "
+                             f"[blocks, {num_kv_heads}, block, {head_dim}]")
+        if kcache.dtype != qkv.dtype or vcache.dtype != qkv.dtype:
+            raise TypeError("qk_norm_rope_cache: the cache has the activations' dtype")
+        _int32(positions, "positions", T)
+        _int32(slots, "cache slots", T)
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() < rotary_dim // 2:
+            raise ValueError("qk_norm_rope_cache: inv_freq is float32 with rotary_dim/2 entries")
+        wtag = 0
+        for w in (q_weight, k_weight):
+            if w is not None:
+                if w.shape != (head_dim,):
+                    raise ValueError(f"qk_norm_rope_cache: head-norm weight {tuple(w.shape)}, expected [{head_dim}]")
+                wtag = _tag(w, "head-norm weight")
+        if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+            raise TypeError("qk_norm_rope_cache: q and k norm weights differ in dtype")
+        library.call("ra_qk_norm_rope_cache", qkv.data_ptr(), _tag(qkv, "qkv"), _ptr(q_weight),
+                     _ptr(k_weight), wtag, float(eps), positions.data_ptr(), inv_freq.data_ptr(),
+                     int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(),
+                     vcache.data_ptr(), kcache.shape[2], T, num_heads, num_kv_heads, head_dim, _stream())
+
+    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+        _dev(gate_up, out)
+        T, I = out.shape
+        if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype \
+                or not gate_up.is_contiguous() or not out.is_contiguous():
+            raise ValueError(f"silu_mul: gate_up {tuple(gate_up.shape)} against out {tuple(out.shape)}")
+        library.call("ra_silu_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I, _stream())
+
+    # ------------------------------------------------------------- attention
+    def attention(self, q: torch.Tensor, q_stride: int, out: torch.Tensor, kcache: torch.Tensor,
+                  vcache: torch.Tensor, batch, num_heads: int, num_kv_heads: int, head_dim: int,
+                  scale: float, window: int, group: int) -> None:
+        """Attention of every token of the step over its request's cache.
+
+        ``q`` is the buffer whose row ``t`` holds the query heads of token t at
+        its start (row stride ``q_stride`` elements); ``batch`` is the step's
+        :class:`reinfer_amd.engine.batch.StepBatch`; ``group`` picks the block
+        tables of the cache group this layer belongs to.
+        """
+        self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                             head_dim, scale, window, group)
+
+    def attention_plain(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
+                        scale, window, group) -> None:
+        _dev(q, out, kcache, vcache)
+        T = batch.num_tokens
+        tables = batch.block_tables[group]
+        if out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+            raise ValueError(f"attention: out {tuple(out.shape)}, expected [{T}, {num_heads * head_dim}]")
+        if q.shape[0] != T or q_stride < num_heads * head_dim or q.stride(0) != q_stride:
+            raise ValueError("attention: query rows do not match the step's tokens")
+        if kcache.dtype != q.dtype or kcache.shape != vcache.shape or kcache.shape[1] != num_kv_heads \
+                or kcache.shape[3] != head_dim:
+            raise ValueError("attention: cache does not match the layer's heads")
+        _int32(tables, "block tables")
+        if tables.dim() != 2 or tables.shape[0] < batch.num_seqs:
+            raise ValueError("attention: one block-table row per request of the step")
+        library.call("ra_attention_plain", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+                     kcache.data_ptr(), vcache.data_ptr(), _tag(q, "attention"), tables.data_ptr(),
+                     tables.shape[1], batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), T,
+                     kcache.shape[2], num_heads, num_kv_heads, head_dim, float(scale), int(window),
+                     _stream())
+
+    # ---------------------------------------------------------------- linear
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor,
+               bias: Optional[torch.Tensor] = None) -> None:
+        """out[M, N] = x[M, K] . weight[N, K]^T (+ bias), float accumulation."""
+        self.linear_plain(x, weight, out, bias)
+
+    def linear_plain(self, x, weight, out, bias=None) -> None:
+        _dev(x, weight, out, bias)
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.shape != (N, K) or out.shape != (M, N) or x.dtype != weight.dtype:
+            raise ValueError(f"linear: x {tuple(x.shape)} {x.dtype}, weight {tuple(weight.shape)} "
+                             f"{weight.dtype}, out {tuple(out.shape)}")
+        if x.stride(1) != 1 or out.stride(1) != 1 or not weight.is_contiguous():
+            raise ValueError("linear: rows must be contiguous")
+        if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype):
+            raise ValueError("linear: bias must be [N] in the weight's dtype")
+        library.call("ra_gemm_plain", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                     _tag(x, "linear input"), _tag(out, "linear output"), M, N, K, x.stride(0),
+                     out.stride(0), _stream())
+
+    # -------------------------------------------------------------- sampling
+    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,
+               positions: torch.Tensor, tokens: torch.Tensor) -> None:
+        _dev(logits, temperature, seeds, positions, tokens)
+        n, V = logits.shape
+        if logits.dtype != torch.float32 or logits.stride(1) != 1:
+            raise TypeError("sample: logits are float32 rows")
+        if temperature.dtype != torch.float32 or seeds.dtype != torch.int64:
+            raise TypeError("sample: temperature float32, seeds int64")
+        _int32(positions, "sample positions", n)
+        _int32(tokens, "sampled tokens", n)
+        if temperature.numel() < n or seeds.numel() < n:
+            raise ValueError("sample: one temperature and seed per row")
+        slices = library.load().ra_sample_slices(V)
+        val = torch.empty((n, slices), dtype=torch.float32, device=logits.device)
+        idx = torch.empty((n, slices), dtype=torch.int32, device=logits.device)
+        library.call("ra_sample", logits.data_ptr(), n, V, logits.stride(0), temperature.data_ptr(),
+                     seeds.data_ptr(), positions.data_ptr(), val.data_ptr(), idx.data_ptr(),
+                     tokens.data_ptr(), _stream())

@@ -1,0 +1,76 @@
+"""A decoder put together from a :class:`ModelSpec`: embedding, blocks in run
+order, final norm, head. It knows no architecture by name; what differs between
+architectures is in the spec and in the parts the spec names.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import kernels
+from ..config.schema import ModelSpec
+from ..parts import KVNeed, LayerCache, StateNeed, lookup
+from ..weights import MATRIX, ParamDecl
+
+
+def declare_params(spec: ModelSpec) -> List[ParamDecl]:
+    """Every tensor the model reads, each once, in a fixed order."""
+    out = [ParamDecl(spec.embed_name, (spec.vocab_size, spec.hidden))]
+    for b in spec.blocks:
+        out += lookup("block", b.kind).declare_params(b)
+    out += lookup("norm", spec.final_norm.kind).declare_params(spec.final_norm, spec.final_norm_name)
+    # a tied model may still carry a head tensor in its file: it is not read
+    out.append(ParamDecl(spec.head_name, (spec.vocab_size, spec.hidden), optional=spec.tie_embeddings))
+    seen = set()
+    for d in out:
+        if d.name in seen:
+            raise ValueError(f"tensor {d.name} is declared twice")
+        seen.add(d.name)
+    return out
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
+                 device: torch.device):
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+        self.embed = weights[spec.embed_name]
+        self.blocks = [lookup("block", b.kind)(b, weights, dtype, device) for b in spec.blocks]
+        self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, weights,
+                                                               spec.final_norm_name, dtype, device)
+        # tied: the embedding matrix is the head (crates/cpu/src/model.rs:218-225)
+        self.head = self.embed if spec.tie_embeddings else weights[spec.head_name]
+        self.run_order = spec.run_order
+
+    def cache_needs(self) -> List[Optional[object]]:
+        """What each run-order entry keeps: KVNeed, StateNeed, or None."""
+        needs: List[Optional[object]] = []
+        for e in self.run_order:
+            mixer = self.blocks[e.block].mixer
+            need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
+            needs.append(need)
+        return needs
+
+    def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]]):
+        """Embedding and all blocks: (residual stream, last addend not yet added)."""
+        ops = kernels.current()
+        resid = torch.empty((batch.num_tokens, self.spec.hidden), dtype=torch.float32, device=self.device)
+        ops.embed(self.embed, batch.token_ids, resid)
+        delta = None
+        for i, e in enumerate(self.run_order):
+            delta = self.blocks[e.block].forward(resid, delta, batch, caches[i])
+        return resid, delta
+
+    def forward(self, batch, caches: Sequence[Optional[LayerCache]]) -> torch.Tensor:
+        """Logits [len(batch.logit_rows), vocab] in float32 for the step's tokens.
+
+        The head runs on the wanted rows only (the reference computes all rows of
+        a prompt and keeps the last, crates/cuda/src/engine.rs:5685-5720)."""
+        resid, delta = self.forward_layers(batch, caches)
+        xn = self.final_norm.add_norm(resid, delta, rows=batch.logit_rows)
+        logits = torch.empty((batch.num_logit_rows, self.spec.vocab_size), dtype=torch.float32,
+                             device=self.device)
+        kernels.current().linear(xn, self.head, logits)
+        return logits

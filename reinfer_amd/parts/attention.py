@@ -1,0 +1,85 @@
+"""Grouped-query attention over the paged cache.
+
+q/k/v projections (one fused product), optional per-head RMSNorm of q and k,
+rotation, cache write, attention over the request's block table, output
+projection. Order and formulas: crates/cuda/src/engine.rs:4090-4281 (decode) and
+:5462-5621 (whole prompt); the reference has separate kernels for head norm,
+rotation, scale and cache write and separate calls for prompts and decoding,
+here one fused kernel and one call serve any mix of both. The scale multiplies
+the float score, not q (the reference scales and re-rounds q, engine.rs:4150-4160).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels
+from ..config.schema import MixerSpec
+from ..weights import MATRIX, VECTOR, ParamDecl
+from .base import KVNeed, LayerCache
+from .registry import lookup, register_mixer
+
+
+@register_mixer("gqa_attention")
+class GroupedQueryAttention:
+    @classmethod
+    def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
+        nq = spec.num_heads * spec.head_dim
+        nkv = spec.num_kv_heads * spec.head_dim
+        out = [ParamDecl(prefix + "q_proj.weight", (nq, spec.hidden)),
+               ParamDecl(prefix + "k_proj.weight", (nkv, spec.hidden)),
+               ParamDecl(prefix + "v_proj.weight", (nkv, spec.hidden)),
+               ParamDecl(prefix + "o_proj.weight", (spec.hidden, nq))]
+        if spec.bias:
+            out += [ParamDecl(prefix + "q_proj.bias", (nq,), init="zeros", role=MATRIX),
+                    ParamDecl(prefix + "k_proj.bias", (nkv,), init="zeros", role=MATRIX),
+                    ParamDecl(prefix + "v_proj.bias", (nkv,), init="zeros", role=MATRIX)]
+        if spec.qk_norm:
+            out += [ParamDecl(prefix + "q_norm.weight", (spec.head_dim,), init="norm", role=VECTOR),
+                    ParamDecl(prefix + "k_norm.weight", (spec.head_dim,), init="norm", role=VECTOR)]
+        return out
+
+    def __init__(self, spec: MixerSpec, weights: Dict[str, torch.Tensor], prefix: str,
+                 dtype: torch.dtype, device: torch.device):
+        if spec.num_heads <= 0 or spec.num_kv_heads <= 0 or spec.num_heads % spec.num_kv_heads:
+            raise ValueError(f"{spec.num_heads} query heads do not divide into {spec.num_kv_heads} groups")
+        self.spec = spec
+        self.dtype = dtype
+        self.num_heads, self.num_kv_heads, self.head_dim = spec.num_heads, spec.num_kv_heads, spec.head_dim
+        self.scale = float(spec.scale)
+        self.window = int(spec.window)
+        self.qkv_width = (spec.num_heads + 2 * spec.num_kv_heads) * spec.head_dim
+        # rows of q, k, v one after the other: stays [out, in], K contiguous
+        self.w_qkv = torch.cat([weights[prefix + "q_proj.weight"], weights[prefix + "k_proj.weight"],
+                                weights[prefix + "v_proj.weight"]], dim=0).contiguous()
+        self.b_qkv = None
+        if spec.bias:
+            self.b_qkv = torch.cat([weights[prefix + "q_proj.bias"], weights[prefix + "k_proj.bias"],
+                                    weights[prefix + "v_proj.bias"]], dim=0).to(dtype).contiguous()
+        self.w_o = weights[prefix + "o_proj.weight"]
+        self.q_norm = weights[prefix + "q_norm.weight"] if spec.qk_norm else None
+        self.k_norm = weights[prefix + "k_norm.weight"] if spec.qk_norm else None
+        self.eps = float(spec.qk_norm_eps)
+        self.position = lookup("position", spec.position.kind)(spec.position, device)
+        if self.position.rotary_dim > spec.head_dim:
+            raise ValueError("the rotated width cannot exceed the head size")
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
+        ops = kernels.current()
+        T = x.shape[0]
+        qkv = torch.empty((T, self.qkv_width), dtype=self.dtype, device=x.device)
+        ops.linear(x, self.w_qkv, qkv, self.b_qkv)
+        slots = batch.slots[cache.group] if cache.writes else batch.no_slots
+        ops.qk_norm_rope_cache(qkv, self.q_norm, self.k_norm, self.eps, batch.positions,
+                               self.position.inv_freq, self.position.rotary_dim, self.position.style,
+                               slots, cache.k, cache.v, self.num_heads, self.num_kv_heads, self.head_dim)
+        attn = torch.empty((T, self.num_heads * self.head_dim), dtype=self.dtype, device=x.device)
+        ops.attention(qkv, self.qkv_width, attn, cache.k, cache.v, batch, self.num_heads,
+                      self.num_kv_heads, self.head_dim, self.scale, self.window, cache.group)
+        out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+        ops.linear(attn, self.w_o, out)
+        return out

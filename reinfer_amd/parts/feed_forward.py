@@ -1,0 +1,45 @@
+"""Dense SwiGLU feed-forward: down( silu(gate(x)) * up(x) ), no bias.
+
+crates/cuda/src/engine.rs:4288-4303; silu(g) = g / (1 + exp(-g))
+(crates/cuda/kernels/dense_kernels.cu:202-213). gate and up are one product
+over rows [gate; up], followed by the fused SiLU-gate kernel.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .. import kernels
+from ..config.schema import FeedForwardSpec
+from ..weights import ParamDecl
+from .registry import register_feed_forward
+
+
+@register_feed_forward("swiglu")
+class SwiGLU:
+    @classmethod
+    def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
+        return [ParamDecl(prefix + "gate_proj.weight", (spec.intermediate, spec.hidden)),
+                ParamDecl(prefix + "up_proj.weight", (spec.intermediate, spec.hidden)),
+                ParamDecl(prefix + "down_proj.weight", (spec.hidden, spec.intermediate))]
+
+    def __init__(self, spec: FeedForwardSpec, weights: Dict[str, torch.Tensor], prefix: str,
+                 dtype: torch.dtype, device: torch.device):
+        self.spec = spec
+        self.dtype = dtype
+        self.w_gate_up = torch.cat([weights[prefix + "gate_proj.weight"],
+                                    weights[prefix + "up_proj.weight"]], dim=0).contiguous()
+        self.w_down = weights[prefix + "down_proj.weight"]
+
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        ops = kernels.current()
+        T = x.shape[0]
+        I = self.spec.intermediate
+        gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
+        ops.linear(x, self.w_gate_up, gu)
+        act = torch.empty((T, I), dtype=self.dtype, device=x.device)
+        ops.silu_mul(gu, act)
+        out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
+        ops.linear(act, self.w_down, out)
+        return out

@@ -1,0 +1,127 @@
+"""A CPU stand-in for the kernel library, for tests of the engine's bookkeeping.
+
+It has the method names and argument meaning of ``reinfer_amd.kernels.ops.HipKernels``
+and computes with torch on the CPU, reading and writing the same paged cache
+through the same index arrays. With it the ``not gpu`` tests can run the step
+function, the cache manager and the scheduler end to end where there is no GPU.
+It is not part of the product and nothing in ``reinfer_amd`` imports it; on a GPU
+box the tests use the real kernels.
+"""
+from __future__ import annotations
+
+import torch
+
+
+class KernelDouble:
+    name = "cpu-double"
+
+    def embed(self, table, ids, out):
+        out.copy_(table[ids.long()].float())
+
+    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
+        if rows is None:
+            if delta is not None:
+                resid.add_(delta.float())
+            x = resid
+        else:
+            x = resid[rows.long()]
+            if delta is not None:
+                x = x + delta[rows.long()].float()
+        rstd = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+        out.copy_((x * rstd * weight.float()).to(out.dtype))
+
+    def qk_norm_rope_cache(self, qkv, q_weight, k_weight, eps, positions, inv_freq, rotary_dim,
+                           rope_style, slots, kcache, vcache, num_heads, num_kv_heads, head_dim):
+        T = qkv.shape[0]
+        d = head_dim
+        u = qkv.view(T, num_heads + 2 * num_kv_heads, d).float()
+        q, k, v = u[:, :num_heads], u[:, num_heads:num_heads + num_kv_heads], u[:, num_heads + num_kv_heads:]
+
+        def norm(x, w):
+            if w is None:
+                return x
+            return x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps) * w.float()
+
+        def rot(x):
+            if rotary_dim == 0:
+                return x
+            half = rotary_dim // 2
+            ang = positions.float()[:, None] * inv_freq[:half].float()[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            out = x.clone()
+            if rope_style == 0:
+                a, b = x[..., :half], x[..., half:rotary_dim]
+                out[..., :half] = a * c - b * s
+                out[..., half:rotary_dim] = a * s + b * c
+            else:
+                a, b = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+                out[..., 0:rotary_dim:2] = a * c - b * s
+                out[..., 1:rotary_dim:2] = a * s + b * c
+            return out
+
+        q = rot(norm(q, q_weight))
+        k = rot(norm(k, k_weight))
+        qkv.view(T, -1, d)[:, :num_heads] = q.to(qkv.dtype)
+        bs = kcache.shape[2]
+        for t in range(T):
+            s = int(slots[t])
+            if s < 0:
+                continue
+            kcache[s // bs, :, s % bs, :] = k[t].to(kcache.dtype)
+            vcache[s // bs, :, s % bs, :] = v[t].to(vcache.dtype)
+
+    def silu_mul(self, gate_up, out):
+        I = out.shape[1]
+        g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
+        out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+    def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
+                  scale, window, group):
+        T = batch.num_tokens
+        bs = kcache.shape[2]
+        tables = batch.block_tables[group]
+        ratio = num_heads // num_kv_heads
+        qh = q[:, :num_heads * head_dim].reshape(T, num_heads, head_dim).float()
+        for t in range(T):
+            seq = int(batch.seq_of_token[t])
+            p = int(batch.positions[t])
+            lo = max(0, p - window + 1) if window > 0 else 0
+            keys = torch.arange(lo, p + 1)
+            blk = tables[seq, keys // bs].long()
+            K = kcache[blk, :, keys % bs, :].float()        # [n, Hkv, d]
+            V = vcache[blk, :, keys % bs, :].float()
+            for a in range(num_heads):
+                s = (K[:, a // ratio, :] @ qh[t, a]) * scale
+                pr = torch.softmax(s, dim=0)
+                out[t, a * head_dim:(a + 1) * head_dim] = (pr @ V[:, a // ratio, :]).to(out.dtype)
+
+    attention_plain = attention
+
+    def linear(self, x, weight, out, bias=None):
+        y = x.float() @ weight.float().T
+        if bias is not None:
+            y = y + bias.float()
+        out.copy_(y.to(out.dtype))
+
+    linear_plain = linear
+
+    def sample(self, logits, temperature, seeds, positions, tokens):
+        from plain_qwen3 import mix64, splitmix64, unit_from_u64
+        import math
+        for r in range(logits.shape[0]):
+            T = float(temperature[r])
+            best, idx = float("-inf"), -1
+            base = splitmix64((int(seeds[r]) & ((1 << 64) - 1)) ^ ((int(positions[r]) * 0x9E3779B97F4A7C15) & ((1 << 64) - 1)))
+            for v, x in enumerate(logits[r].tolist()):
+                if not math.isfinite(x):
+                    continue
+                if T > 0:
+                    u = unit_from_u64(mix64(base ^ mix64(v)))
+                    if u <= 0:
+                        continue
+                    x = torch.tensor(x, dtype=torch.float32) / torch.tensor(T, dtype=torch.float32) \
+                        - torch.log(-torch.log(torch.tensor(u, dtype=torch.float32)))
+                    x = float(x)
+                if x > best:
+                    best, idx = x, v
+            tokens[r] = idx

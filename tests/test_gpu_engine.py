@@ -1,0 +1,142 @@
+"""The engine on the GPU against the plain implementation, in 32-bit and bfloat16:
+whole requests, most in one step and the last 32 tokens one by one, portions of
+changing size, mixed batches with page reuse, long decoding, the first tokens.
+The logits at a position must not depend on how the tokens were cut into steps,
+on what else is in the batch or on which blocks are used, beyond rounding."""
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import TINY, TOL, make_folder, mixed_plan, random_tokens, read_folder, rel_err, run_plan
+from reinfer_amd import kernels
+from reinfer_amd.engine import ModelRunner, StepEntry
+
+pytestmark = pytest.mark.gpu
+
+CASES = [(w, d) for w in ("A", "B", "C") for d in ("float32", "bfloat16")]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    return {(w, d): make_folder(base, w, d) for w, d in CASES}
+
+
+@pytest.fixture(scope="module")
+def plain_cache():
+    return {}
+
+
+def reference(folders, plain_cache, which, dtype, toks):
+    key = (which, dtype, tuple(toks))
+    if key not in plain_cache:
+        raw, weights = read_folder(folders[(which, dtype)])
+        plain_cache[key] = plain.forward(raw, weights, toks).float()
+    return plain_cache[key]
+
+
+def runner_for(folders, which, dtype, **limits):
+    assert kernels.current().name == "hip-gfx950"
+    return ModelRunner.from_folder(folders[(which, dtype)], dtype=dtype, device="cuda:0", **limits)
+
+
+def vocab(which):
+    return TINY[which][0]["vocab_size"]
+
+
+@pytest.mark.parametrize("which,dtype", CASES)
+def test_whole(folders, plain_cache, which, dtype):
+    runner = runner_for(folders, which, dtype, max_tokens=256)
+    for n, seed in ((5, 1), (17, 2), (33, 3), (130, 4), (1, 5)):
+        toks = random_tokens(n, vocab(which), seed)
+        got = run_plan(runner, {"r": toks}, [[("r", n)]])["r"]
+        assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype], (n,)
+    assert all(p.num_free == p.num_blocks for p in runner.manager.pools)
+
+
+@pytest.mark.parametrize("which,dtype", CASES)
+def test_last_32_one_by_one(folders, plain_cache, which, dtype):
+    runner = runner_for(folders, which, dtype, max_tokens=256)
+    n = 150
+    toks = random_tokens(n, vocab(which), 21)
+    plan = [[("r", n - 32)]] + [[("r", 1)]] * 32
+    got = run_plan(runner, {"r": toks}, plan)["r"]
+    assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("which,dtype", CASES)
+def test_portions_of_changing_size(folders, plain_cache, which, dtype):
+    runner = runner_for(folders, which, dtype, max_tokens=256)
+    n = 131
+    toks = random_tokens(n, vocab(which), 22)
+    cuts = [7, 2, 16, 3, 2, 17, 2, 31, 2, 15, 1, 16, 2, 2, 13]
+    assert sum(cuts) == n
+    got = run_plan(runner, {"r": toks}, [[("r", c)] for c in cuts])["r"]
+    assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("which,dtype", CASES)
+def test_mixed_with_page_reuse(folders, plain_cache, which, dtype):
+    runner = runner_for(folders, which, dtype, max_tokens=128)
+    lens, plan = mixed_plan()
+    seqs = {r: random_tokens(n, vocab(which), 300 + i) for i, (r, n) in enumerate(lens.items())}
+    # poison everything a request does not own: a read outside its blocks shows as NaN
+    for c in runner.caches:
+        if c is not None and c.k is not None:
+            c.k.fill_(float("nan"))
+            c.v.fill_(float("nan"))
+    got = run_plan(runner, seqs, plan)
+    for r, toks in seqs.items():
+        assert rel_err(got[r], reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype], r
+    pool = runner.manager.pools[0]
+    assert pool.allocs > pool.num_blocks, "the plan must reuse blocks"
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_long_decoding(folders, plain_cache, which, dtype):
+    runner = runner_for(folders, which, dtype, max_tokens=256)
+    n = 200
+    toks = random_tokens(n, vocab(which), 23)
+    got = run_plan(runner, {"r": toks}, [[("r", 3)]] + [[("r", 1)]] * (n - 3))["r"]
+    assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("which,dtype", CASES)
+def test_first_tokens(folders, plain_cache, which, dtype):
+    """Positions 0, 1, 2 on their own: one key, two keys; page edges at 15/16/17."""
+    runner = runner_for(folders, which, dtype, max_tokens=64)
+    toks = random_tokens(18, vocab(which), 24)
+    ref = reference(folders, plain_cache, which, dtype, toks)
+    got = run_plan(runner, {"r": toks}, [[("r", 1)]] * 18)["r"]
+    assert rel_err(got[:3], ref[:3]) < TOL[dtype]
+    assert rel_err(got, ref) < TOL[dtype]
+
+
+def test_far_key_stands_out(folders):
+    """One early key that a late query must find among hundreds: a fault in the
+    block table walk or in the running maximum would lose it. The query and key
+    weights of the first layer are scaled so that scores are sharp."""
+    which, dtype = "B", "float32"
+    raw, weights = read_folder(folders[(which, dtype)])
+    weights = {k: v.clone() for k, v in weights.items()}
+    for name in ("q_norm", "k_norm"):
+        weights[f"model.layers.0.self_attn.{name}.weight"] *= 3.0
+    from reinfer_amd.config import config_from_dict
+    runner = ModelRunner.from_config(config_from_dict(raw), dtype=dtype, weights=weights, max_tokens=512)
+    toks = random_tokens(400, raw["vocab_size"], 25)
+    ref = plain.forward(raw, weights, toks).float()
+    plan = [[("r", 2)], [("r", 333)], [("r", 2)]] + [[("r", 1)]] * 63
+    got = run_plan(runner, {"r": toks}, plan)["r"]
+    assert rel_err(got, ref) < TOL[dtype]
+
+
+def test_batch_order_does_not_matter(folders):
+    runner = runner_for(folders, "A", "float32", max_tokens=256)
+    V = vocab("A")
+    seqs = {"x": random_tokens(30, V, 31), "y": random_tokens(9, V, 32), "z": random_tokens(17, V, 33)}
+    a = run_plan(runner, seqs, [[("x", 30), ("y", 9), ("z", 17)]])
+    b = run_plan(runner, seqs, [[("z", 17), ("x", 30), ("y", 9)]])
+    alone = {r: run_plan(runner, {r: t}, [[(r, len(t))]])[r] for r, t in seqs.items()}
+    for r in seqs:
+        assert rel_err(a[r], alone[r]) < 1e-5
+        assert rel_err(b[r], alone[r]) < 1e-5
