@@ -282,13 +282,13 @@ def test_linear_plain(M, N, K, din, dout):
 
 
 def test_float32_linear_is_true_float32():
-    """Values that a reduced-precision matrix mode would round away survive."""
-    K = 64
-    x = torch.ones(1, K, device=DEV)
-    w = torch.full((1, K), 1.0 + 2.0 ** -20, device=DEV)      # not representable in 16 or 19 bits
+    """(1 + 2^-12)^2 - 1 = 2^-11 + 2^-24: inputs rounded to 10 or 7 mantissa bits give 0."""
+    a = 1.0 + 2.0 ** -12
+    x = torch.tensor([[a, 1.0]], device=DEV)
+    w = torch.tensor([[a, -1.0]], device=DEV)
     out = torch.empty(1, 1, device=DEV)
     ops().linear_plain(x, w, out)
-    assert abs(out.item() - K * (1.0 + 2.0 ** -20)) < 1e-5
+    assert abs(out.item() - (2.0 ** -11 + 2.0 ** -24)) < 1e-7     # float rounding of a*a itself
 
 
 # -------------------------------------------------------------- sampling
