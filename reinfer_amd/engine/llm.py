@@ -1,0 +1,144 @@
+"""The Python entry point: model folder (or configuration + seed) to generated tokens.
+
+    engine = LLMEngine("path/to/model")                    # or LLMEngine(config=cfg, seed=0)
+    outs = engine.generate([[1, 2, 3], [4, 5]], SamplingParams(max_tokens=16))
+
+``generate`` runs the scheduler loop: admit, cut prompts into portions under the
+token budget, decode, sample on the GPU, finish and free. ``add_request`` /
+``step`` / ``abort`` expose the same loop one step at a time, ``step_raw`` is the
+step function itself (what trace replay drives). The reference's single-request
+loop is bin/reinfer/src/pipeline.rs:123-239 and its batching loop
+bin/reinfer/src/sched_loop.rs:691-1029; it re-runs the last prompt token as the
+first decode step (pipeline.rs:173-178), here the first token is sampled from
+the logits at the prompt's last position.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config import load_config
+from ..sampling import Sampler, SamplingParams, derive_seed
+from .batch import StepEntry
+from .runner import ModelRunner
+from .scheduler import FINISHED, Request, RequestRefused, Scheduler, StepPlan
+
+
+@dataclass
+class RequestOutput:
+    rid: Hashable
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: Optional[str]
+    preemptions: int = 0
+
+
+class LLMEngine:
+    def __init__(self, model: Optional[str] = None, *, config=None, seed: int = 0,
+                 dtype: str = "bfloat16", device: str = "cuda:0", weights=None,
+                 max_model_len: Optional[int] = None, block_size: int = 16,
+                 num_blocks: Optional[int] = None, max_num_seqs: int = 64,
+                 max_num_batched_tokens: int = 2048, max_chunk: Optional[int] = None,
+                 memory_fraction: float = 0.9):
+        limits = dict(block_size=block_size, num_blocks=num_blocks, max_seqs=max_num_seqs,
+                      max_model_len=max_model_len, memory_fraction=memory_fraction)
+        if model is not None:
+            self.config = load_config(model)
+            self.runner = ModelRunner.from_folder(model, dtype=dtype, device=device, **limits)
+        elif config is not None:
+            self.config = config
+            self.runner = ModelRunner.from_config(config, seed=seed, dtype=dtype, device=device,
+                                                  weights=weights, **limits)
+        else:
+            raise ValueError("give a model folder, or a configuration (random weights from the seed)")
+        self.seed = int(seed)
+        self.device = self.runner.device
+        self.scheduler = Scheduler(self.runner.manager, max_num_seqs=max_num_seqs,
+                                   max_num_batched_tokens=max_num_batched_tokens,
+                                   max_model_len=self.runner.max_model_len, max_chunk=max_chunk,
+                                   eos_token_ids=self.runner.spec.eos_token_ids)
+        self.sampler = Sampler(self.device)
+        self._auto_id = 0
+        self.timings: Dict[str, float] = {}
+
+    # --------------------------------------------------------- requests
+    def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    rid: Optional[Hashable] = None) -> Hashable:
+        params = params or SamplingParams()
+        if rid is None:
+            rid = f"req-{self._auto_id}"
+            self._auto_id += 1
+        V = self.runner.spec.vocab_size
+        for t in prompt_token_ids:
+            if not 0 <= int(t) < V:
+                raise RequestRefused(f"token {t} outside the vocabulary of {V}")
+        arrival = self.scheduler._arrivals
+        seed = params.seed if params.seed is not None else derive_seed(self.seed, arrival)
+        self.scheduler.add(rid, prompt_token_ids, params, seed)
+        return rid
+
+    def abort(self, rid: Hashable) -> bool:
+        return self.scheduler.abort(rid)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # -------------------------------------------------------------- step
+    def step(self) -> List[RequestOutput]:
+        """One scheduler decision, one batch through the model, one sampling call."""
+        plan = self.scheduler.schedule()
+        finished = [self._output(r) for r in plan.finished]
+        if not plan.portions:
+            if not finished and self.scheduler.has_work() and not plan.preempted:
+                raise RuntimeError("the scheduler could place no token although work is waiting")
+            return finished
+        entries, rows = [], []
+        for p in plan.portions:
+            toks = p.request.tokens[p.start:p.start + p.length]
+            entries.append(StepEntry(p.request.rid, toks, [p.length - 1] if p.samples else []))
+            if p.samples:
+                rows.append(p.request)
+        logits = self.runner.step(entries)
+        sampled: Dict[Hashable, int] = {}
+        if rows:
+            toks = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
+                                       [r.num_tokens for r in rows], [r.tokens for r in rows])
+            sampled = {r.rid: t for r, t in zip(rows, toks)}
+        done = self.scheduler.complete(plan, sampled)
+        return finished + [self._output(r) for r in done]
+
+    @staticmethod
+    def _output(r: Request) -> RequestOutput:
+        return RequestOutput(r.rid, list(r.prompt), list(r.output), r.finish_reason, r.preemptions)
+
+    def step_raw(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """The step function itself: given tokens in, float32 logits out, no sampling."""
+        return self.runner.step(entries)
+
+    # ---------------------------------------------------------- generate
+    def generate(self, prompt_token_ids: Sequence[Sequence[int]],
+                 sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None
+                 ) -> List[RequestOutput]:
+        if isinstance(sampling_params, SamplingParams) or sampling_params is None:
+            sampling_params = [sampling_params or SamplingParams()] * len(prompt_token_ids)
+        if len(sampling_params) != len(prompt_token_ids):
+            raise ValueError("one SamplingParams per prompt")
+        rids = [self.add_request(p, sp) for p, sp in zip(prompt_token_ids, sampling_params)]
+        outs: Dict[Hashable, RequestOutput] = {}
+        t0 = time.perf_counter()
+        first = None
+        while self.scheduler.has_work():
+            for o in self.step():
+                outs[o.rid] = o
+            if first is None:
+                first = time.perf_counter() - t0
+        self.timings = {"total_s": time.perf_counter() - t0, "first_step_s": first or 0.0}
+        return [outs[r] for r in rids]
+
+    def cache_stats(self) -> Dict[str, object]:
+        s = self.runner.manager.stats()
+        s.update(self.scheduler.counters)
+        return s

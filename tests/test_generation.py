@@ -1,0 +1,122 @@
+"""Generation through the Python entry point and the command line: greedy equals the
+plain implementation, preemption does not change outputs, seeded temperature
+sampling does not depend on the batch. The CPU runs use the kernel stand-in
+(bookkeeping only); the ``gpu`` runs use the real kernels."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import TINY, make_folder, random_tokens, read_folder
+from kernel_double import KernelDouble
+from reinfer_amd import LLMEngine, SamplingParams, kernels
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def engine_for(folder, device, dtype="float32", **kw):
+    return LLMEngine(folder, dtype=dtype, device=device, **kw)
+
+
+def check_greedy(folder, device):
+    raw, w = read_folder(folder)
+    prompts = [random_tokens(n, raw["vocab_size"], 40 + n) for n in (5, 17, 33)]
+    want = [plain.greedy_generate(raw, w, p, 16) for p in prompts]
+    eng = engine_for(folder, device, num_blocks=32)
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16))
+    assert [o.token_ids for o in outs] == want
+    assert all(o.finish_reason == "length" for o in outs)
+    # so few blocks that requests are preempted and recomputed: the same tokens
+    small = engine_for(folder, device, num_blocks=6, max_num_batched_tokens=24)
+    outs2 = small.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16))
+    assert [o.token_ids for o in outs2] == want
+    assert small.cache_stats()["preemptions"] > 0
+    assert small.cache_stats()["blocks_free"] == small.cache_stats()["blocks_total"]
+    return eng
+
+
+def check_temperature(folder, device):
+    raw, w = read_folder(folder)
+    V = raw["vocab_size"]
+    prompts = [random_tokens(n, V, 70 + n) for n in (1, 7, 64, 130)]
+    sp = [SamplingParams(temperature=0.8, seed=1000 + i, max_tokens=12) for i in range(len(prompts))]
+    eng = engine_for(folder, device, num_blocks=64, max_num_batched_tokens=16)    # portions of 16 beside decodes
+    together = [o.token_ids for o in eng.generate(prompts, sp)]
+    again = [o.token_ids for o in eng.generate(prompts, sp)]
+    assert together == again, "same seed, same tokens"
+    alone = [eng.generate([p], s)[0].token_ids for p, s in zip(prompts, sp)]
+    assert alone == together, "a request's tokens do not depend on the batch"
+    other = eng.generate(prompts[:1], SamplingParams(temperature=0.8, seed=5, max_tokens=12))[0].token_ids
+    assert other != together[0]
+    assert all(0 <= t < V for o in together for t in o)
+
+
+def test_greedy_generation_cpu_bookkeeping(tmp_path):
+    with kernels.use(KernelDouble()):
+        check_greedy(make_folder(tmp_path, "A", "float32"), "cpu")
+
+
+def test_temperature_generation_cpu_bookkeeping(tmp_path):
+    with kernels.use(KernelDouble()):
+        check_temperature(make_folder(tmp_path, "B", "float32"), "cpu")
+
+
+def test_eos_from_config_stops_generation(tmp_path):
+    with kernels.use(KernelDouble()):
+        folder = make_folder(tmp_path, "A", "float32")
+        raw, w = read_folder(folder)
+        prompt = random_tokens(6, raw["vocab_size"], 5)
+        free_run = plain.greedy_generate(raw, w, prompt, 6)
+        raw2 = dict(raw, eos_token_id=free_run[3])
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(raw2, f)
+        out = engine_for(folder, "cpu", num_blocks=16).generate([prompt], SamplingParams(max_tokens=6))[0]
+        cut = free_run.index(free_run[3])
+        assert out.token_ids == free_run[:cut] and out.finish_reason == "stop"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_greedy_generation_gpu(tmp_path, which):
+    eng = check_greedy(make_folder(tmp_path, which, "float32"), "cuda:0")
+    assert kernels.current().name == "hip-gfx950"
+
+
+@pytest.mark.gpu
+def test_temperature_generation_gpu(tmp_path):
+    check_temperature(make_folder(tmp_path, "B", "float32"), "cuda:0")
+
+
+@pytest.mark.gpu
+def test_bfloat16_greedy_mostly_agrees_with_plain(tmp_path):
+    """bfloat16 may flip a near tie; where the plain top-2 gap is clear the tokens agree."""
+    folder = make_folder(tmp_path, "B", "bfloat16")
+    raw, w = read_folder(folder)
+    prompt = random_tokens(20, raw["vocab_size"], 9)
+    out = engine_for(folder, "cuda:0", dtype="bfloat16", num_blocks=32).generate(
+        [prompt], SamplingParams(max_tokens=12))[0].token_ids
+    toks = list(prompt)
+    for t in out:
+        logits = plain.forward(raw, w, toks)[-1]
+        top2 = torch.topk(logits, 2).values
+        if (top2[0] - top2[1]) > 0.05 * logits.abs().max():
+            assert t == int(torch.argmax(logits))
+        toks.append(t)
+
+
+@pytest.mark.gpu
+def test_command_line_run(tmp_path):
+    folder = make_folder(tmp_path, "A", "float32")
+    raw, w = read_folder(folder)
+    prompt = [3, 141, 59, 26, 53]
+    want = plain.greedy_generate(raw, w, prompt, 8)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "reinfer"), "run", folder, "-n", "8", "-t", "0",
+                        "--dtype", "float32", "--num-blocks", "16", "--perf", "--"] + [str(t) for t in prompt],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [int(t) for t in r.stdout.split()] == want
+    assert "PERF " in r.stderr and "tok_s=" in r.stderr and "first_token_ms=" in r.stderr

@@ -1,0 +1,128 @@
+"""The plain implementation, pinned by what fixes it beside the reference's text:
+vectors the reference's own tests hold, special cases that reduce to a library
+routine, and invariants, each chosen so that a plausible mistake fails it."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import TINY_A, TINY_B, make_folder, random_tokens, read_folder
+
+D = torch.float64
+
+
+def test_rms_norm_vectors():
+    """crates/kernels/src/refs.rs:168-178: [3,4] with w=[1,2], eps 0 -> [3,8]/sqrt(12.5); zero row -> 0."""
+    y = plain.rms_norm(torch.tensor([3.0, 4.0], dtype=D), torch.tensor([1.0, 2.0], dtype=D), 0.0)
+    assert torch.allclose(y, torch.tensor([3.0, 8.0], dtype=D) / math.sqrt(12.5))
+    z = plain.rms_norm(torch.zeros(4, dtype=D), torch.ones(4, dtype=D), 1e-6)
+    assert torch.equal(z, torch.zeros(4, dtype=D))
+    # eps sits inside the root: a norm with eps outside gives 1/(0 + 1e-3), not 1/sqrt(1e-3)
+    x = torch.full((8,), 1e-9, dtype=D)
+    assert abs(plain.rms_norm(x, torch.ones(8, dtype=D), 1e-6)[0].item() - 1e-9 / math.sqrt(1e-18 + 1e-6)) < 1e-15
+    # against the library routine
+    x = torch.randn(5, 33, dtype=D)
+    w = torch.rand(33, dtype=D)
+    assert torch.allclose(plain.rms_norm(x, w, 1e-5), torch.nn.functional.rms_norm(x, (33,), w, 1e-5))
+
+
+def test_head_norm_is_per_head():
+    u = torch.randn(3, 4, 16, dtype=D)
+    y = plain.head_norm(u, torch.ones(16, dtype=D), 0.0)
+    assert torch.allclose((y * y).mean(dim=-1), torch.ones(3, 4, dtype=D))     # every head has RMS 1
+    # a norm over all heads together would not
+    u2 = u.clone()
+    u2[:, 0] *= 10
+    y2 = plain.head_norm(u2, torch.ones(16, dtype=D), 0.0)
+    assert torch.allclose(y2[:, 1:], y[:, 1:])
+
+
+def test_rope_vectors_and_invariants():
+    """crates/kernels/src/refs.rs:181-192: position 0 is the identity; pair norms are
+    kept for half=3, pos=7, theta=5000."""
+    x = torch.tensor([[[1.0, -2.0, 0.5, 3.0, 0.25, -1.5]]], dtype=D)
+    assert torch.allclose(plain.rope_neox(x, torch.tensor([0]), 5000.0), x)
+    y = plain.rope_neox(x, torch.tensor([7]), 5000.0)
+    for j in range(3):
+        assert abs((y[0, 0, j] ** 2 + y[0, 0, j + 3] ** 2) - (x[0, 0, j] ** 2 + x[0, 0, j + 3] ** 2)) < 1e-12
+    # the pairing is (j, j + half), and the sign: a complex multiplication by e^{i phi}
+    d, pos, theta = 8, 5, 100.0
+    u = torch.randn(1, 1, d, dtype=D)
+    z = torch.complex(u[..., :4], u[..., 4:]) * torch.polar(
+        torch.ones(4, dtype=D), pos * theta ** (-2.0 * torch.arange(4, dtype=D) / d))
+    got = plain.rope_neox(u, torch.tensor([pos]), theta)
+    assert torch.allclose(got[..., :4], z.real) and torch.allclose(got[..., 4:], z.imag)
+    # only distances count
+    q, k = torch.randn(1, 1, 16, dtype=D), torch.randn(1, 1, 16, dtype=D)
+    def dot(p, t):
+        return (plain.rope_neox(q, torch.tensor([p]), 1e4) * plain.rope_neox(k, torch.tensor([t]), 1e4)).sum()
+    assert abs(dot(9, 4) - dot(109, 104)) < 1e-10
+    assert abs(dot(9, 4) - dot(4, 9)) > 1e-6      # but the sign of the distance does
+
+
+def test_attention_reduces_to_library_and_masks():
+    T, H, d = 9, 3, 8
+    q, k, v = (torch.randn(T, H, d, dtype=D) for _ in range(3))
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+    assert torch.allclose(plain.causal_attention(q, k, v, 1 / math.sqrt(d)), ref)
+    # grouped: query head a reads KV head a // ratio (14/2, 12/2: crates/cuda/tests/gqa_diff.rs:1-16)
+    for Hq, Hkv in ((14, 2), (12, 2), (4, 4), (8, 1)):
+        q = torch.randn(T, Hq, d, dtype=D)
+        k, v = torch.randn(T, Hkv, d, dtype=D), torch.randn(T, Hkv, d, dtype=D)
+        r = Hq // Hkv
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            q.transpose(0, 1)[None], k.repeat_interleave(r, 1).transpose(0, 1)[None],
+            v.repeat_interleave(r, 1).transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+        assert torch.allclose(plain.causal_attention(q, k, v, 1 / math.sqrt(d)), ref)
+    # one key: the output is its value; later keys never leak into earlier rows
+    out = plain.causal_attention(q, k, v, 0.3)
+    assert torch.allclose(out[0, 0], v[0, 0])
+    k2, v2 = k.clone(), v.clone()
+    k2[5:], v2[5:] = 99.0, -99.0
+    assert torch.allclose(plain.causal_attention(q, k2, v2, 0.3)[:5], out[:5])
+    # a window of W keeps keys p-W+1..p
+    w3 = plain.causal_attention(q, k, v, 0.3, window=3)
+    k3, v3 = k.clone(), v.clone()
+    k3[:4], v3[:4] = 50.0, 50.0                   # positions 0..3 are outside the window of row 6
+    assert torch.allclose(plain.causal_attention(q, k3, v3, 0.3, window=3)[6:], w3[6:])
+    assert torch.allclose(plain.causal_attention(q, k, v, 0.3, window=T), out)
+
+
+def test_swiglu():
+    x = torch.randn(4, 6, dtype=D)
+    wg, wu, wd = torch.randn(10, 6, dtype=D), torch.randn(10, 6, dtype=D), torch.randn(6, 10, dtype=D)
+    F = torch.nn.functional
+    assert torch.allclose(plain.swiglu(x, wg, wu, wd), F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd))
+    assert torch.equal(plain.swiglu(x, torch.zeros_like(wg), wu, wd), torch.zeros(4, 6, dtype=D))   # gate 0 -> 0
+
+
+def test_whole_model_special_cases(tmp_path):
+    raw, w = read_folder(make_folder(tmp_path, "B", "float32"))
+    toks = random_tokens(12, raw["vocab_size"], 1)
+    full = plain.forward(raw, w, toks)
+    # with the output and down projections zero, logits = head(norm(embedding))
+    w0 = {k: (torch.zeros_like(v) if ("o_proj" in k or "down_proj" in k) else v) for k, v in w.items()}
+    x = w["model.embed_tokens.weight"][torch.tensor(toks)].double()
+    want = plain.rms_norm(x, w["model.norm.weight"].double(), raw["rms_norm_eps"]) @ w["lm_head.weight"].double().T
+    assert torch.allclose(plain.forward(raw, w0, toks), want)
+    # causal: a prefix's logits do not depend on what follows
+    assert torch.allclose(plain.forward(raw, w, toks[:7]), full[:7])
+    # a shift of all positions changes nothing (only distances count)
+    assert torch.allclose(plain.forward(raw, w, toks, start_pos=37), full, atol=1e-9)
+    # tied = untied with the head set to the embedding
+    rawA, wA = read_folder(make_folder(tmp_path, "A", "float32"))
+    toksA = random_tokens(9, rawA["vocab_size"], 2)
+    untied = dict(rawA, tie_word_embeddings=False)
+    wA2 = dict(wA)
+    wA2["lm_head.weight"] = wA["model.embed_tokens.weight"]
+    assert torch.equal(plain.forward(rawA, wA, toksA), plain.forward(untied, wA2, toksA))
+
+
+def test_splitmix_vectors_and_greedy_ties():
+    """crates/scheduler/src/rng.rs:83-87."""
+    assert plain.splitmix64(0) == 0xE220A8397B1DCDAF
+    assert plain.splitmix64(1) == 0x910A2DEC89025CC1
+    assert plain.unit_from_u64((1 << 64) - 1) < 1.0 and plain.unit_from_u64(0) == 0.0
+    assert plain.argmax_first(torch.tensor([1.0, 5.0, 5.0, 2.0])) == 1      # first maximum

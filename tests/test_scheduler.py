@@ -1,0 +1,228 @@
+"""The scheduler's decisions, without a model: a fake step whose sampled token is a
+pure function of (request, position), as the reference's MockExecutor does
+(bin/reinfer/src/sched_loop.rs:1594-1776)."""
+import pytest
+
+import plain_qwen3 as plain
+from reinfer_amd.cache import CacheGroupSpec, CacheManager
+from reinfer_amd.engine.scheduler import FINISHED, RUNNING, WAITING, RequestRefused, Scheduler
+from reinfer_amd.sampling import SamplingParams
+
+
+def make(num_blocks=64, bs=4, max_seqs=8, budget=32, max_model_len=512, max_chunk=None, eos=(), windows=(0,)):
+    groups = [CacheGroupSpec(window=w, entries=(i,)) for i, w in enumerate(windows)]
+    m = CacheManager(groups, bs, [num_blocks] * len(groups), max_seqs)
+    s = Scheduler(m, max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_model_len,
+                  max_chunk=max_chunk, eos_token_ids=eos)
+    return m, s
+
+
+def fake_token(rid, position, vocab=1000):
+    return plain.splitmix64(hash(str(rid)) % (1 << 32) * 7919 + position) % vocab
+
+
+def run_step(m, s, log=None, token_fn=fake_token):
+    plan = s.schedule()
+    assert plan.num_tokens <= s.budget
+    for p in plan.portions:
+        assert p.start == p.request.num_computed, "a portion starts where the cache ends"
+        m.grow(p.request.rid, p.start + p.length)
+    for p in plan.portions:
+        m.commit(p.request.rid, p.start + p.length)
+    sampled = {p.request.rid: token_fn(p.request.rid, p.request.num_tokens) for p in plan.portions if p.samples}
+    if log is not None:
+        log.append(([(p.request.rid, p.start, p.length) for p in plan.portions],
+                    [r.rid for r in plan.preempted]))
+    done = s.complete(plan, sampled)
+    m.check()
+    return plan, done
+
+
+def drive(m, s, log=None, limit=10000, token_fn=fake_token):
+    outs = {}
+    n = 0
+    while s.has_work():
+        plan, done = run_step(m, s, log, token_fn)
+        for r in done + plan.finished:
+            outs[r.rid] = (list(r.output), r.finish_reason)
+        n += 1
+        assert n < limit, "the scheduler does not terminate"
+    return outs
+
+
+def test_decode_first_then_portion_under_budget():
+    """batch.rs:128-142 with an effective budget of 8: three decoders take 3, the
+    prompt of 40 gets [0, 5)."""
+    m, s = make(budget=8, max_chunk=16)
+    for i in range(3):
+        s.add(f"d{i}", [1, 2], SamplingParams(max_tokens=50), seed=i)
+    run_step(m, s)                              # prompts of 2 tokens each: 6 tokens
+    assert all(r.decoding for r in s.running)
+    s.add("p", list(range(40)), SamplingParams(max_tokens=5), seed=9)
+    plan, _ = run_step(m, s)
+    got = [(p.request.rid, p.start, p.length) for p in plan.portions]
+    assert got == [("d0", 2, 1), ("d1", 2, 1), ("d2", 2, 1), ("p", 0, 5)]
+    # continuation starts at the computed length (batch.rs:174-179)
+    plan, _ = run_step(m, s)
+    assert ("p", 5, 5) in [(p.request.rid, p.start, p.length) for p in plan.portions]
+
+
+def test_max_chunk_and_fcfs():
+    m, s = make(budget=64, max_chunk=16)
+    s.add("a", list(range(40)), SamplingParams(max_tokens=2), seed=0)
+    s.add("b", list(range(10)), SamplingParams(max_tokens=2), seed=0)
+    plan, _ = run_step(m, s)
+    assert [(p.request.rid, p.start, p.length) for p in plan.portions] == [("a", 0, 16), ("b", 0, 10)]
+    plan, _ = run_step(m, s)        # b decodes, a continues
+    assert [(p.request.rid, p.start, p.length) for p in plan.portions] == [("a", 16, 16), ("b", 10, 1)]
+
+
+def test_exactly_max_tokens_and_stop_ids():
+    m, s = make()
+    s.add("a", [5, 6, 7], SamplingParams(max_tokens=7), seed=0)
+    outs = drive(m, s)
+    assert len(outs["a"][0]) == 7 and outs["a"][1] == "length"
+    # an end-of-sequence id is consumed, not emitted (req.rs:281-314)
+    m, s = make(eos=(42,))
+    s.add("a", [1], SamplingParams(max_tokens=20), seed=0)
+    seq = iter([3, 4, 42, 5])
+    outs = drive(m, s, token_fn=lambda rid, pos: next(seq))
+    assert outs["a"] == ([3, 4], "stop")
+    m, s = make(eos=(42,))
+    s.add("a", [1], SamplingParams(max_tokens=4, ignore_eos=True, stop_token_ids=(5,)), seed=0)
+    seq = iter([3, 42, 5, 6])
+    assert drive(m, s, token_fn=lambda rid, pos: next(seq))["a"] == ([3, 42], "stop")
+
+
+def test_context_limit_ends_a_request():
+    m, s = make(max_model_len=10)
+    s.add("a", [1] * 6, SamplingParams(max_tokens=100), seed=0)
+    outs = drive(m, s)
+    assert len(outs["a"][0]) == 4 and outs["a"][1] == "length"      # 6 + 4 = 10 tokens
+    with pytest.raises(RequestRefused, match="context"):
+        s.add("b", [1] * 10, SamplingParams(), seed=0)
+
+
+def test_refusals():
+    m, s = make(num_blocks=4, bs=4)             # 16 tokens of cache
+    with pytest.raises(RequestRefused, match="empty"):
+        s.add("a", [], SamplingParams(), seed=0)
+    with pytest.raises(RequestRefused, match="never fit"):
+        s.add("a", [1] * 16, SamplingParams(), seed=0)
+    s.add("a", [1] * 15, SamplingParams(max_tokens=1), seed=0)
+    with pytest.raises(RequestRefused, match="already live"):
+        s.add("a", [1], SamplingParams(), seed=0)
+    assert s.counters["refused"] == 2
+
+
+def test_preemption_newest_first_and_same_output():
+    """Pages run out while decoding: the newest arrival is preempted, goes to the
+    head of the queue, is recomputed, and ends with the output it would have had."""
+    def run(num_blocks):
+        m, s = make(num_blocks=num_blocks, bs=4, budget=64, max_seqs=4)
+        for i, n in enumerate([9, 7, 8]):
+            s.add(f"r{i}", list(range(1, n + 1)), SamplingParams(max_tokens=30), seed=i)
+        log = []
+        outs = drive(m, s, log)
+        assert all(p.num_free == p.num_blocks for p in m.pools)
+        return outs, log, s
+    big, _, s_big = run(64)
+    small, log, s_small = run(16)               # 64 tokens of cache for 3 x ~39
+    assert s_big.counters["preemptions"] == 0 and s_small.counters["preemptions"] > 0
+    assert small == big
+    first = next(pre for _, pre in log if pre)
+    assert first[0] == "r2", "the newest arrival goes first (policy.rs:59-63)"
+    # a resumed request restarts at position 0 with prompt + generated tokens
+    step_after = next(i for i, (_, pre) in enumerate(log) if pre)
+    resumed = [x for portions, _ in log[step_after + 1:] for x in portions if x[0] == "r2"][0]
+    assert resumed[1] == 0
+    assert s_small.requests["r2"].preemptions >= 1 and s_small.requests["r2"].resumed
+
+
+def test_resumed_requests_are_preempted_last():
+    m, s = make(num_blocks=64, bs=4, max_seqs=4)
+    for i in range(3):
+        s.add(f"r{i}", [1, 2, 3], SamplingParams(max_tokens=50), seed=i)
+    run_step(m, s)
+    s.requests["r2"].resumed = True
+    victims = sorted(s.running, key=lambda r: (r.resumed, -r.arrival))
+    assert [r.rid for r in victims] == ["r1", "r0", "r2"]
+
+
+def test_lone_request_that_outgrows_the_cache_ends():
+    m, s = make(num_blocks=3, bs=4)             # 12 tokens
+    s.add("a", [1] * 5, SamplingParams(max_tokens=100), seed=0)
+    outs = drive(m, s)
+    assert outs["a"][1] == "cache" and len(outs["a"][0]) == 8      # 5 + 7 fill the 12 slots; the 8th token has no slot
+    assert all(p.num_free == p.num_blocks for p in m.pools)
+
+
+def test_abort_is_idempotent_and_isolated():
+    def run(abort):
+        m, s = make()
+        for i in range(3):
+            s.add(f"r{i}", [i + 1] * 5, SamplingParams(max_tokens=12), seed=i)
+        run_step(m, s)
+        run_step(m, s)
+        if abort:
+            assert s.abort("r1") and not s.abort("r1") and not s.abort("nobody")
+            assert s.requests["r1"].finish_reason == "abort"
+        outs = drive(m, s)
+        m.check()
+        assert all(p.num_free == p.num_blocks for p in m.pools)
+        return outs
+    with_abort, without = run(True), run(False)
+    assert "r1" not in with_abort
+    assert with_abort["r0"] == without["r0"] and with_abort["r2"] == without["r2"]
+    # aborting a waiting request
+    m, s = make(max_seqs=1)
+    s.add("a", [1], SamplingParams(max_tokens=3), seed=0)
+    s.add("b", [1], SamplingParams(max_tokens=3), seed=0)
+    assert s.abort("b") and s.requests["b"].state == FINISHED
+    assert set(drive(m, s)) == {"a"}
+
+
+def test_max_num_seqs_caps_running():
+    m, s = make(max_seqs=2)
+    for i in range(5):
+        s.add(f"r{i}", [1, 2], SamplingParams(max_tokens=3), seed=i)
+    while s.has_work():
+        run_step(m, s)
+        assert len(s.running) <= 2
+    assert s.counters["finished"] == 5
+
+
+def test_admission_keeps_headroom_for_running_requests():
+    m, s = make(num_blocks=6, bs=4, budget=64)
+    s.add("a", [1] * 8, SamplingParams(max_tokens=20), seed=0)
+    run_step(m, s)                              # a holds 2 blocks (+1 at its next token)
+    s.add("b", [1] * 16, SamplingParams(max_tokens=2), seed=0)
+    plan, _ = run_step(m, s)
+    # 4 blocks free, a takes 1, one stays in reserve for a: b gets 2 blocks = 8 tokens now
+    assert [(p.request.rid, p.start, p.length) for p in plan.portions] == [("a", 8, 1), ("b", 0, 8)]
+
+
+def test_replay_twice_is_identical():
+    """A fixed arrival list decides the same twice (crates/scheduler/src/replay.rs:171-177)."""
+    def run(seed):
+        import random
+        rng = random.Random(seed)
+        m, s = make(num_blocks=24, bs=4, budget=24, max_seqs=4, windows=(0, 6))
+        arrivals = [(rng.randrange(0, 30), [rng.randrange(1, 99) for _ in range(rng.randrange(1, 30))],
+                     rng.randrange(1, 20)) for _ in range(12)]
+        log, outs, step, i = [], {}, 0, 0
+        arrivals.sort(key=lambda a: a[0])
+        while i < len(arrivals) or s.has_work():
+            while i < len(arrivals) and arrivals[i][0] <= step:
+                s.add(f"r{i}", arrivals[i][1], SamplingParams(max_tokens=arrivals[i][2]), seed=i)
+                i += 1
+            if s.has_work():
+                plan, done = run_step(m, s, log)
+                for r in done + plan.finished:
+                    outs[r.rid] = (list(r.output), r.finish_reason)
+            step += 1
+            assert step < 5000
+        assert all(p.num_free == p.num_blocks for p in m.pools)
+        return log, outs
+    for seed in range(5):
+        assert run(seed) == run(seed)
