@@ -43,7 +43,7 @@ def _add_run_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
     p.add_argument("--prompt-len", type=int, default=None, metavar="N",
                    help="use N seeded random token ids as the prompt")
-    p.add_argument("prompt", nargs=argparse.REMAINDER, help="prompt: token ids, or text with a tokenizer.json")
+    p.add_argument("prompt", nargs="*", help="prompt: token ids, or text with a tokenizer.json")
 
 
 def _load_tokenizer(model_dir: str):
