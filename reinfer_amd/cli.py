@@ -43,7 +43,6 @@ def _add_run_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
     p.add_argument("--prompt-len", type=int, default=None, metavar="N",
                    help="use N seeded random token ids as the prompt")
-    p.add_argument("prompt", nargs="*", help="prompt: token ids, or text with a tokenizer.json")
 
 
 def _load_tokenizer(model_dir: str):
@@ -145,7 +144,19 @@ def main(argv: Optional[List[str]] = None) -> int:
     p = sub.add_parser("bench", help="throughput measurement (see bench.py --help)")
     p.add_argument("rest", nargs=argparse.REMAINDER)
     p.set_defaults(fn=cmd_bench)
-    args = ap.parse_args(argv)
+    argv = list(sys.argv[1:] if argv is None else argv)
+    # the prompt is what follows "--", else the trailing words no option takes
+    # (the reference's trailing_var_arg, bin/reinfer/src/main.rs:290-292)
+    prompt: List[str] = []
+    if "--" in argv:
+        cut = argv.index("--")
+        argv, prompt = argv[:cut], argv[cut + 1:]
+    args, extra = ap.parse_known_args(argv)
+    if extra:
+        if args.verb not in ("run", "generate") or any(w.startswith("-") and not w.lstrip("-").isdigit() for w in extra):
+            ap.error("unrecognized arguments: " + " ".join(extra))
+        prompt = extra + prompt
+    args.prompt = prompt
     return args.fn(args)
 
 
