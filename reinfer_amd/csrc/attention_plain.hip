@@ -17,6 +17,7 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
                                        int out_stride, const TA* __restrict__ kcache,
                                        const TA* __restrict__ vcache,
                                        const int* __restrict__ block_tables, int max_blocks,
+                                       const int* __restrict__ token_list,
                                        const int* __restrict__ seq_of_token,
                                        const int* __restrict__ positions, int block_size, int Hq,
                                        int Hkv, int d, float scale, int window) {
@@ -25,7 +26,7 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
   float* ps = lds + d;
   const int lane = threadIdx.x;
   const int a = blockIdx.x;
-  const int t = blockIdx.y;
+  const int t = token_list ? token_list[blockIdx.y] : blockIdx.y;
   const int kvh = a / (Hq / Hkv);
   const int seq = seq_of_token[t];
   const int p = positions[t];
@@ -91,8 +92,8 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
 
 extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride,
                                   const void* kcache, const void* vcache, int act_dtype,
-                                  const int* block_tables, int max_blocks, const int* seq_of_token,
-                                  const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
+                                  const int* block_tables, int max_blocks, const int* token_list,
+                                  const int* seq_of_token, const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
                                   int d, float scale, int window, hipStream_t stream) {
   RA_CHECK(n_tokens > 0, "attention_plain: no tokens");
   RA_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "attention_plain: %d query heads do not divide into %d groups", Hq, Hkv);
@@ -105,12 +106,12 @@ extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int ou
   if (act_dtype == RA_F32)
     attention_plain_kernel<float><<<grid, RA_WAVE, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)kcache, (const float*)vcache,
-        block_tables, max_blocks, seq_of_token, positions, block_size, Hq, Hkv, d, scale, window);
+        block_tables, max_blocks, token_list, seq_of_token, positions, block_size, Hq, Hkv, d, scale, window);
   else if (act_dtype == RA_BF16)
     attention_plain_kernel<bf16_t><<<grid, RA_WAVE, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-        (const bf16_t*)vcache, block_tables, max_blocks, seq_of_token, positions, block_size, Hq, Hkv,
-        d, scale, window);
+        (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size,
+        Hq, Hkv, d, scale, window);
   else
     return ra_fail("attention_plain: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("attention_plain");

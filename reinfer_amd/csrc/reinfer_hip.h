@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 1
+#define RA_ABI_VERSION 2
 
 #ifdef __cplusplus
 extern "C" {
@@ -30,11 +30,35 @@ int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int
 
 int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                        const void* vcache, int act_dtype, const int* block_tables, int max_blocks,
-                       const int* seq_of_token, const int* positions, int n_tokens, int block_size,
+                       const int* token_list, const int* seq_of_token, const int* positions, int n_tokens,
+                       int block_size,
                        int Hq, int Hkv, int d, float scale, int window, hipStream_t stream);
 
 int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int in_dtype, int out_dtype,
                   int M, int N, int K, int lda, int ldc, hipStream_t stream);
+
+// bfloat16, M <= 64, K and lda multiples of 8: weight-streaming MFMA product
+int ra_gemm_skinny_max_rows(void);
+int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int M, int N,
+                   int K, int lda, int ldc, hipStream_t stream);
+
+// bfloat16 flash-decode: one query per listed token, split-KV; partial buffers are
+// float [n_tokens, Hq, n_splits, d] and [n_tokens, Hq, n_splits, 2] (unused for one split)
+int ra_attention_decode_supports(int Hq, int Hkv, int d);
+int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                        const void* vcache, const int* block_tables, int max_blocks,
+                        const int* token_list, const int* seq_of_token, const int* positions,
+                        int n_tokens, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                        int n_splits, float* part_o, float* part_ml, hipStream_t stream);
+
+// bfloat16 flash prefill over query tiles; tile_info holds 4 ints per tile:
+// request row in block_tables, first token row, number of queries (<= tile), first position
+int ra_attention_prefill_supports(int Hq, int Hkv, int d);
+int ra_attention_prefill_tile(void);
+int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                         const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
+                         int n_tiles, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                         hipStream_t stream);
 
 int ra_sample_slices(int vocab);
 int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,

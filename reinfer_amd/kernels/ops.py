@@ -129,6 +129,8 @@ class HipKernels:
         library.call("ra_silu_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I, _stream())
 
     # ------------------------------------------------------------- attention
+    SHORT_PORTION = 4     # portions up to this many tokens go token by token through the decode kernel
+
     def attention(self, q: torch.Tensor, q_stride: int, out: torch.Tensor, kcache: torch.Tensor,
                   vcache: torch.Tensor, batch, num_heads: int, num_kv_heads: int, head_dim: int,
                   scale: float, window: int, group: int) -> None:
@@ -137,13 +139,68 @@ class HipKernels:
         ``q`` is the buffer whose row ``t`` holds the query heads of token t at
         its start (row stride ``q_stride`` elements); ``batch`` is the step's
         :class:`reinfer_amd.engine.batch.StepBatch`; ``group`` picks the block
-        tables of the cache group this layer belongs to.
+        tables of the cache group this layer belongs to. bfloat16: single tokens
+        and short portions take the split-KV decode kernel, longer portions the
+        MFMA prefill kernel in tiles of queries; sizes neither takes, and
+        float32, go to the plain kernel.
         """
-        self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                             head_dim, scale, window, group)
+        lib = library.load()
+        if q.dtype != torch.bfloat16:
+            return self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                        head_dim, scale, window, group)
+        plan = self._attention_plan(batch, q.device)
+        dec_ok = bool(lib.ra_attention_decode_supports(num_heads, num_kv_heads, head_dim))
+        pre_ok = bool(lib.ra_attention_prefill_supports(num_heads, num_kv_heads, head_dim))
+        if plan["n_decode"]:
+            if dec_ok:
+                self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                      head_dim, scale, window, group, plan["decode_list"], plan["n_decode"],
+                                      plan["decode_max_ctx"])
+            else:
+                self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                     head_dim, scale, window, group, plan["decode_list"], plan["n_decode"])
+        if plan["n_tiles"]:
+            if pre_ok:
+                self.attention_prefill(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                       head_dim, scale, window, group, plan["tiles"], plan["n_tiles"])
+            else:
+                self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                     head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"])
 
-    def attention_plain(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
-                        scale, window, group) -> None:
+    def _attention_plan(self, batch, device):
+        """Which tokens go to which kernel; made once per step, shared by the layers."""
+        plan = batch.extra.get("attention_plan")
+        if plan is not None:
+            return plan
+        tile = library.load().ra_attention_prefill_tile()
+        dec, pre, tiles = [], [], []
+        dec_max_ctx = 0
+        t = 0
+        for i, (ql, st) in enumerate(zip(batch.q_lens, batch.starts)):
+            if ql <= self.SHORT_PORTION:
+                dec.extend(range(t, t + ql))
+                dec_max_ctx = max(dec_max_ctx, st + ql)
+            else:
+                pre.extend(range(t, t + ql))
+                for q0 in range(0, ql, tile):
+                    tiles.extend((i, t + q0, min(tile, ql - q0), st + q0))
+            t += ql
+        all_decode = len(dec) == batch.num_tokens
+        flat = ([] if all_decode else dec) + pre + tiles
+        dev = torch.tensor(flat, dtype=torch.int32).to(device, non_blocking=True) if flat else None
+        n_dec_listed = 0 if all_decode else len(dec)
+        plan = {
+            "n_decode": len(dec), "decode_max_ctx": dec_max_ctx,
+            "decode_list": None if all_decode or not dec else dev[:n_dec_listed],
+            "n_prefill": len(pre),
+            "prefill_list": dev[n_dec_listed:n_dec_listed + len(pre)] if pre else None,
+            "n_tiles": len(tiles) // 4,
+            "tiles": dev[n_dec_listed + len(pre):] if tiles else None,
+        }
+        batch.extra["attention_plan"] = plan
+        return plan
+
+    def _check_attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim, group):
         _dev(q, out, kcache, vcache)
         T = batch.num_tokens
         tables = batch.block_tables[group]
@@ -152,24 +209,92 @@ class HipKernels:
         if q.shape[0] != T or q_stride < num_heads * head_dim or q.stride(0) != q_stride:
             raise ValueError("attention: query rows do not match the step's tokens")
         if kcache.dtype != q.dtype or kcache.shape != vcache.shape or kcache.shape[1] != num_kv_heads \
-                or kcache.shape[3] != head_dim:
+                or kcache.shape[3] != head_dim or not kcache.is_contiguous() or not vcache.is_contiguous():
             raise ValueError("attention: cache does not match the layer's heads")
         _int32(tables, "block tables")
         if tables.dim() != 2 or tables.shape[0] < batch.num_seqs:
             raise ValueError("attention: one block-table row per request of the step")
+        # every key a query may read must have a table entry
+        if tables.shape[1] * kcache.shape[2] < batch.max_ctx_len:
+            raise ValueError("attention: block tables shorter than the longest context")
+        return tables
+
+    def attention_plain(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
+                        scale, window, group, token_list=None, n_listed=None) -> None:
+        tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                       head_dim, group)
+        n = batch.num_tokens if token_list is None else int(n_listed)
         library.call("ra_attention_plain", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), _tag(q, "attention"), tables.data_ptr(),
-                     tables.shape[1], batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), T,
+                     tables.shape[1], _ptr(token_list), batch.seq_of_token.data_ptr(),
+                     batch.positions.data_ptr(), n, kcache.shape[2], num_heads, num_kv_heads, head_dim,
+                     float(scale), int(window), _stream())
+
+    @staticmethod
+    def decode_splits(n_tokens: int, num_kv_heads: int, max_ctx: int) -> int:
+        """Split-KV factor: enough workgroups to fill 256 CUs a few times over, and
+        at least 256 keys a split."""
+        want = -(-1024 // max(1, n_tokens * num_kv_heads))
+        return max(1, min(want, max(1, max_ctx // 256), 64))
+
+    def attention_decode(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
+                         scale, window, group, token_list=None, n_listed=None, max_ctx=None,
+                         n_splits=None) -> None:
+        tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                       head_dim, group)
+        if q.dtype != torch.bfloat16:
+            raise TypeError("attention_decode: bfloat16 only")
+        n = batch.num_tokens if token_list is None else int(n_listed)
+        if n_splits is None:
+            n_splits = self.decode_splits(n, num_kv_heads, max_ctx or batch.max_ctx_len)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty((n, num_heads, n_splits, head_dim), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((n, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
+        library.call("ra_attention_decode", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+                     kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
+                     _ptr(token_list), batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), n,
                      kcache.shape[2], num_heads, num_kv_heads, head_dim, float(scale), int(window),
-                     _stream())
+                     int(n_splits), _ptr(part_o), _ptr(part_ml), _stream())
+
+    def attention_prefill(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
+                          scale, window, group, tiles, n_tiles) -> None:
+        tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
+                                       head_dim, group)
+        if q.dtype != torch.bfloat16:
+            raise TypeError("attention_prefill: bfloat16 only")
+        _int32(tiles, "query tiles", 4 * n_tiles)
+        library.call("ra_attention_prefill", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+                     kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
+                     tiles.data_ptr(), int(n_tiles), kcache.shape[2], num_heads, num_kv_heads, head_dim,
+                     float(scale), int(window), _stream())
 
     # ---------------------------------------------------------------- linear
     def linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor,
                bias: Optional[torch.Tensor] = None) -> None:
-        """out[M, N] = x[M, K] . weight[N, K]^T (+ bias), float accumulation."""
+        """out[M, N] = x[M, K] . weight[N, K]^T (+ bias), float accumulation.
+
+        bfloat16 with up to 64 rows: the weight-streaming MFMA kernel. bfloat16
+        with more rows and a bfloat16 result: the library product (hipBLASLt
+        through torch), as the reference calls cuBLAS for its prompt products
+        (crates/cuda/src/gemm.rs:226-292). Everything else, all of float32
+        included: the plain FMA kernel.
+        """
+        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+            M, K = x.shape
+            if M <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1:
+                return self.linear_skinny(x, weight, out, bias)
+            if out.dtype == torch.bfloat16 and x.is_cuda:
+                self._check_linear(x, weight, out, bias)
+                if bias is None:
+                    torch.mm(x, weight.t(), out=out)
+                else:
+                    torch.addmm(bias, x, weight.t(), out=out)
+                return
         self.linear_plain(x, weight, out, bias)
 
-    def linear_plain(self, x, weight, out, bias=None) -> None:
+    @staticmethod
+    def _check_linear(x, weight, out, bias):
         _dev(x, weight, out, bias)
         M, K = x.shape
         N = weight.shape[0]
@@ -180,9 +305,20 @@ class HipKernels:
             raise ValueError("linear: rows must be contiguous")
         if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype):
             raise ValueError("linear: bias must be [N] in the weight's dtype")
+        return M, N, K
+
+    def linear_plain(self, x, weight, out, bias=None) -> None:
+        M, N, K = self._check_linear(x, weight, out, bias)
         library.call("ra_gemm_plain", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                      _tag(x, "linear input"), _tag(out, "linear output"), M, N, K, x.stride(0),
                      out.stride(0), _stream())
+
+    def linear_skinny(self, x, weight, out, bias=None) -> None:
+        M, N, K = self._check_linear(x, weight, out, bias)
+        if x.dtype != torch.bfloat16:
+            raise TypeError("linear_skinny: bfloat16 only")
+        library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                     _tag(out, "linear output"), M, N, K, x.stride(0), out.stride(0), _stream())
 
     # -------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,

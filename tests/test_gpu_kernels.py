@@ -362,3 +362,140 @@ def test_sample_distribution_is_softmax():
     p = torch.softmax(row.double() / T, dim=0)
     # 4 standard deviations of a binomial frequency
     assert ((freq - p).abs() <= 4 * torch.sqrt(p * (1 - p) / n) + 1e-4).all(), (freq, p)
+
+
+# ------------------------------------------------- bfloat16 kernels of serving
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("N,K", [(100, 64), (333, 136), (1000, 96), (6144, 4096), (257, 520), (16, 8)])
+@pytest.mark.parametrize("dout", ["bfloat16", "float32"])
+def test_linear_skinny(M, N, K, dout):
+    torch.manual_seed(M * N + K)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV).to(torch.bfloat16)
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=DT[dout])
+    ops().linear_skinny(x, w, out)
+    ref = x.double() @ w.double().T
+    close(out, ref, OUT_TOL[dout])
+    ops().linear_skinny(x, w, out, b)
+    close(out, ref + b.double(), OUT_TOL[dout])
+    # the row of a token does not depend on its neighbours: row r of the batch = the single-row product
+    one = torch.empty(1, N, device=DEV, dtype=DT[dout])
+    ops().linear_skinny(x[M - 1:M], w, one)
+    ops().linear_skinny(x, w, out)
+    close(one, out[M - 1:M], 1e-6 if dout == "float32" else 2 ** -8)
+
+
+def test_linear_dispatch_refuses_nothing_silently():
+    """Sizes the MFMA kernel does not take go to the plain kernel, not to a wrong result."""
+    x = torch.randn(5, 100, device=DEV).to(torch.bfloat16)[:, :99]       # K = 99, odd row stride
+    w = torch.randn(7, 99, device=DEV).to(torch.bfloat16)
+    out = torch.empty(5, 7, device=DEV, dtype=torch.bfloat16)
+    ops().linear(x, w, out)
+    close(out, x.double() @ w.double().T, 2 ** -8)
+    with pytest.raises(kernels.KernelLibraryError, match="multiples of 8"):
+        ops().linear_skinny(x.contiguous(), w, out)
+    big = torch.randn(65, 64, device=DEV).to(torch.bfloat16)
+    with pytest.raises(kernels.KernelLibraryError, match="at most 64"):
+        ops().linear_skinny(big, torch.randn(8, 64, device=DEV).to(torch.bfloat16),
+                            torch.empty(65, 8, device=DEV, dtype=torch.bfloat16))
+
+
+DEC_SHAPES = [(4, 2, 16), (14, 2, 64), (12, 2, 48), (5, 5, 32), (8, 1, 128), (32, 8, 128), (2, 1, 256), (6, 3, 80)]
+DEC_BATCHES = [
+    ([1], [0]), ([1], [15]), ([1], [16]), ([1, 1, 1], [31, 32, 700]), ([1] * 5, [63, 64, 65, 1000, 2]),
+    ([2, 1, 3, 1], [0, 257, 30, 99]),
+]
+
+
+@pytest.mark.parametrize("Hq,Hkv,d", DEC_SHAPES)
+def test_attention_decode(Hq, Hkv, d):
+    for bi, (q_lens, starts) in enumerate(DEC_BATCHES):
+        for window in (0, 19):
+            for n_splits in (1, 3, 8):
+                q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=10 + bi)
+                batch = FakeBatch(q_lens, starts, tables)
+                T = sum(q_lens)
+                out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+                scale = 1.0 / math.sqrt(d)
+                ops().attention_decode(q.view(T, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hkv, d, scale, window, 0,
+                                       n_splits=n_splits)
+                ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
+                close(out, ref, 2 ** -7)     # probabilities and values are bfloat16 products summed in float
+
+
+def test_attention_decode_token_list_leaves_other_rows_alone():
+    Hq, Hkv, d = 8, 2, 64
+    q_lens, starts = [1, 6, 1], [40, 3, 99]
+    q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=3)
+    batch = FakeBatch(q_lens, starts, tables)
+    T = sum(q_lens)
+    out = torch.full((T, Hq * d), 7.0, device=DEV, dtype=torch.bfloat16)
+    lst = torch.tensor([0, 7], dtype=torch.int32, device=DEV)
+    ops().attention_decode(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0, lst, 2, 100)
+    ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0)
+    close(out[[0, 7]], ref[[0, 7]], 2 ** -7)
+    assert (out[1:7] == 7.0).all()
+
+
+PRE_BATCHES = [
+    ([5], [0]), ([64], [0]), ([65], [0]), ([17, 130], [30, 5]), ([200], [0]), ([33, 7, 64], [1, 700, 16]),
+    ([300], [213]),
+]
+
+
+@pytest.mark.parametrize("Hq,Hkv,d", [(4, 2, 16), (14, 2, 64), (12, 2, 48), (5, 5, 32), (8, 1, 128), (32, 8, 128),
+                                      (6, 3, 80), (3, 1, 112)])
+def test_attention_prefill(Hq, Hkv, d):
+    tile = 64
+    for bi, (q_lens, starts) in enumerate(PRE_BATCHES):
+        for window in (0, 19, 100):
+            q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=20 + bi)
+            batch = FakeBatch(q_lens, starts, tables)
+            T = sum(q_lens)
+            out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+            info, t = [], 0
+            for i, (ql, st) in enumerate(zip(q_lens, starts)):
+                for q0 in range(0, ql, tile):
+                    info += [i, t + q0, min(tile, ql - q0), st + q0]
+                t += ql
+            tiles = torch.tensor(info, dtype=torch.int32, device=DEV)
+            scale = 1.0 / math.sqrt(d)
+            ops().attention_prefill(q.view(T, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hkv, d, scale, window, 0,
+                                    tiles, len(info) // 4)
+            ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
+            close(out, ref, 2 ** -7)
+
+
+def test_attention_dispatch_mixed_batch():
+    """Single tokens, a short portion and long portions in one call: each token gets
+    the kernel its portion calls for, and every row is written once."""
+    Hq, Hkv, d = 8, 2, 64
+    q_lens, starts = [1, 3, 70, 1, 5], [100, 0, 11, 15, 64]
+    q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=9)
+    batch = FakeBatch(q_lens, starts, tables)
+    T = sum(q_lens)
+    out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().attention(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0)
+    plan = batch.extra["attention_plan"]
+    assert plan["n_decode"] == 5 and plan["n_tiles"] == 3
+    close(out, attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0), 2 ** -7)
+
+
+def test_far_key_among_hundreds_decode_and_prefill():
+    """One key far back matches the query much better than all others: losing it
+    (a wrong block, a dropped split, a wrong running maximum) changes the output."""
+    Hq, Hkv, d = 4, 1, 128
+    for q_lens, starts in (([1], [900]), ([80], [821])):
+        q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=4)
+        far = 37
+        blk = int(tables[0, far // 16])
+        kc[blk, 0, far % 16] = (q[-1, 0].float() * 3).to(torch.bfloat16)      # the last query's first head points at it
+        vc[blk, 0, far % 16] = 5.0
+        batch = FakeBatch(q_lens, starts, tables)
+        T = sum(q_lens)
+        out = torch.empty((T, Hq * d), device=DEV, dtype=torch.bfloat16)
+        ops().attention(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0)
+        ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0)
+        assert ref[-1, :d].mean() > 4.0           # the far value dominates the reference
+        close(out, ref, 2 ** -7)
