@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+The default run is the Qwen3-8B shape (36 layers, width 4096, 32 query heads over
+8 KV heads of 128, feed-forward 12288, vocabulary 151936, separate head) in
+bfloat16 with random weights N(0, 0.02) and uniform-random prompts: 8 requests
+with 2,048-token prompts are prefilled, then W untimed and K timed decode steps
+run through the engine's own loop (scheduler, step function, GPU sampler). One
+JSON line goes to standard output: ``value`` is decoded tokens a second at batch
+8; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the
+decode step against 8 TB/s by the bytes it must read (every weight once and the
+keys and values of the live requests); ``points`` holds batch 1 and batch 64.
+The reference publishes no number at this size (its own are Qwen3-0.6B on a
+laptop GPU, bench/gate-fixture.md:66-74), so ``vs_baseline`` is null.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12                       # bytes a second
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_8B = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": 36,
+    "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 4096, "attention_bias": False,
+}
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def linear_params(raw: dict) -> int:
+    """Matrix elements a token passes through: layers and head (the embedding is a row read)."""
+    h, L = raw["hidden_size"], raw["num_hidden_layers"]
+    nq = raw["num_attention_heads"] * raw["head_dim"]
+    nkv = raw["num_key_value_heads"] * raw["head_dim"]
+    per_layer = h * (nq + 2 * nkv) + nq * h + 3 * h * raw["intermediate_size"]
+    return L * per_layer + raw["vocab_size"] * h
+
+
+def kv_bytes_per_token(raw: dict, elem: int) -> int:
+    return 2 * raw["num_hidden_layers"] * raw["num_key_value_heads"] * raw["head_dim"] * elem
+
+
+def decode_run(engine, raw, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps. -> (ms a step, mean context)."""
+    import torch
+    from reinfer_amd.sampling import SamplingParams
+    g = torch.Generator().manual_seed(seed)
+    params = SamplingParams(temperature=0.0, max_tokens=raw["max_position_embeddings"] - prompt_len - 1,
+                            ignore_eos=True)
+    rids = []
+    for _ in range(batch):
+        ids = torch.randint(0, raw["vocab_size"], (prompt_len,), generator=g).tolist()
+        rids.append(engine.add_request(ids, params))
+    sched = engine.scheduler
+    # prompts first: until every request is decoding
+    while any(not r.decoding for r in sched.running) or sched.waiting:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    ctx0 = statistics.mean(r.num_tokens for r in sched.running)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert len(sched.running) == batch, "a request ended inside the timed steps"
+    ctx1 = statistics.mean(r.num_tokens for r in sched.running)
+    for r in rids:
+        engine.abort(r)
+    return dt * 1e3 / steps, 0.5 * (ctx0 + ctx1)
+
+
+def prefill_run(engine, raw, tokens: int, reps: int, seed: int) -> float:
+    """Median milliseconds of one ``tokens``-long prompt run as one step (its first token sampled)."""
+    import torch
+    from reinfer_amd.sampling import SamplingParams
+    g = torch.Generator().manual_seed(seed)
+    times = []
+    for i in range(reps + 2):
+        ids = torch.randint(0, raw["vocab_size"], (tokens,), generator=g).tolist()
+        rid = engine.add_request(ids, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.abort(rid)
+        if i >= 2:
+            times.append(dt * 1e3)
+    return statistics.median(times)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from reinfer_amd import kernels
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.engine import LLMEngine
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    kernels.current()
+    raw = dict(QWEN3_8B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(raw)
+    ctx_len = raw["max_position_embeddings"]
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    block = 16
+    # a request decodes while later prompts are still being prefilled: one step a prompt
+    blocks_per_req = -(-(args.prompt_len + max_batch + args.warmup + args.steps + 16) // block)
+    num_blocks = max_batch * blocks_per_req + 8
+    log(f"building {raw['num_hidden_layers']} layers of the Qwen3-8B shape in {args.dtype}, random weights ...")
+    t0 = time.perf_counter()
+    engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=block, num_blocks=num_blocks,
+                       max_num_seqs=max_batch, max_num_batched_tokens=max(2048, args.prefill_tokens),
+                       max_model_len=ctx_len)
+    torch.cuda.synchronize()
+    log(f"model ready in {time.perf_counter() - t0:.1f} s; {num_blocks} cache blocks of {block}")
+
+    elem = 2 if args.dtype == "bfloat16" else 4
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    n_lin = linear_params(raw)
+    kv_tok = kv_bytes_per_token(raw, elem)
+
+    # prefill: one prompt, one step
+    T = args.prefill_tokens
+    pf_ms = prefill_run(engine, raw, T, reps=5, seed=args.seed + 1)
+    nq = raw["num_attention_heads"] * raw["head_dim"]
+    # every row through every matrix but the head (one row), causal attention (scores and values)
+    pf_flops = 2.0 * (n_lin - raw["vocab_size"] * raw["hidden_size"]) * T + 2.0 * raw["vocab_size"] * raw["hidden_size"] \
+        + 2.0 * nq * T * T * raw["num_hidden_layers"]
+    prefill = {"value": round(T / (pf_ms * 1e-3), 1), "tokens": T, "ms": round(pf_ms, 3),
+               "frac": round(pf_flops / (pf_ms * 1e-3) / MFMA_PEAK[dkey], 4)}
+    log(f"prefill {T} tokens: {pf_ms:.2f} ms, {prefill['value']:.0f} tok/s, {prefill['frac']:.3f} of the MFMA peak")
+
+    ms, ctx = decode_run(engine, raw, args.batch, args.prompt_len, args.steps, args.warmup, args.seed + 2)
+    value = args.batch / (ms * 1e-3)
+    step_bytes = n_lin * elem + args.batch * ctx * kv_tok
+    achieved = step_bytes / (ms * 1e-3)
+    log(f"decode batch {args.batch}: {ms:.3f} ms a step, {value:.0f} tok/s, {achieved / 1e9:.0f} GB/s")
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            steps_b = args.steps if b == 1 else max(16, args.steps // 2)
+            pms, _ = decode_run(engine, raw, b, args.prompt_len, steps_b, min(args.warmup, 16), args.seed + 3 + b)
+            points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
+            log(f"decode batch {b}: {pms:.3f} ms a step, {points[f'decode_b{b}']:.0f} tok/s")
+
+    out = {
+        "metric": "decode tok/s at batch 8 (Qwen3-8B shape, bf16, 2048-token prompts)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dkey, "data": "synthetic (uniform-random token ids, random weights N(0, 0.02))",
+        "config": {
+            "model": "Qwen3-8B shape", "layers": raw["num_hidden_layers"], "layers_of_model": full_layers,
+            "hidden": raw["hidden_size"], "q_heads": raw["num_attention_heads"],
+            "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
+            "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"],
+            "tied_head": raw["tie_word_embeddings"], "global_batch": args.batch, "seq_len": ctx_len,
+            "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "block_size": block,
+            "parallelism": "single GPU",
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
