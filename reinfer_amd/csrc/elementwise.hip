@@ -212,32 +212,38 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
 }
 
 // ---------------------------------------------------------------------------
-// SiLU gate: out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g / (1 + exp(-g))
-// (crates/cuda/kernels/dense_kernels.cu:202-213)
+// SiLU gate: out[t, i] = silu(g[t, i]) * u[t, i], silu(g) = g / (1 + exp(-g))
+// (crates/cuda/kernels/dense_kernels.cu:202-213). gate_up is [T, 2I]; with
+// group == 0 gate is columns [0, I) and up [I, 2I); with group > 0 the two are
+// interleaved in runs of `group` columns, as the gated product kernel wants them.
 // ---------------------------------------------------------------------------
 template <typename TA>
-__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, size_t total) {
+__global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; idx < total; idx += stride) {
     const size_t t = idx / I;
     const int i = (int)(idx - t * I);
-    const float g = to_f32(gu[t * 2 * I + i]);
-    const float u = to_f32(gu[t * 2 * I + I + i]);
+    const size_t gi = group > 0 ? (size_t)(i / group) * 2 * group + i % group : (size_t)i;
+    const size_t ui = group > 0 ? gi + group : (size_t)I + i;
+    const float g = to_f32(gu[t * 2 * I + gi]);
+    const float u = to_f32(gu[t * 2 * I + ui]);
     out[idx] = from_f32<TA>(g / (1.f + expf(-g)) * u);
   }
 }
 
 extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
-                           hipStream_t stream) {
+                           int group, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && intermediate > 0, "silu_mul: empty input");
+  RA_CHECK(group >= 0 && (group == 0 || intermediate % group == 0),
+           "silu_mul: width %d is not a whole number of runs of %d", intermediate, group);
   const size_t total = (size_t)n_tokens * intermediate;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   if (act_dtype == RA_F32)
-    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, total);
+    silu_mul_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total);
   else if (act_dtype == RA_BF16)
-    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, total);
+    silu_mul_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total);
   else
     return ra_fail("silu_mul: unknown dtype tag %d", act_dtype);
   RA_LAUNCH_CHECK("silu_mul");

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 2
+#define RA_ABI_VERSION 3
 
 #ifdef __cplusplus
 extern "C" {
@@ -25,8 +25,10 @@ int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const 
                           int rotary_dim, int rope_style, const int* slots, void* kcache, void* vcache,
                           int block_size, int n_tokens, int Hq, int Hkv, int d, hipStream_t stream);
 
+// gate_up is [T, 2I]: group == 0: gate columns [0, I), up columns [I, 2I); group > 0: gate and
+// up interleaved in runs of `group` columns (gate run, then the up run of the same features)
 int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
-                hipStream_t stream);
+                int group, hipStream_t stream);
 
 int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                        const void* vcache, int act_dtype, const int* block_tables, int max_blocks,
@@ -37,10 +39,12 @@ int ra_attention_plain(const void* q, int q_stride, void* out, int out_stride, c
 int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int in_dtype, int out_dtype,
                   int M, int N, int K, int lda, int ldc, hipStream_t stream);
 
-// bfloat16, M <= 64, K and lda multiples of 8: weight-streaming MFMA product
+// bfloat16, M <= 64, K and lda multiples of 8: weight-streaming MFMA product.
+// epilogue 0: C[M, N] = A . W^T (+ bias); epilogue 1: W rows are gate/up interleaved in runs of 8
+// and C[M, N/2] = silu(gate) * up
 int ra_gemm_skinny_max_rows(void);
-int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int M, int N,
-                   int K, int lda, int ldc, hipStream_t stream);
+int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
+                   int M, int N, int K, int lda, int ldc, hipStream_t stream);
 
 // bfloat16 flash-decode: one query per listed token, split-KV; partial buffers are
 // float [n_tokens, Hq, n_splits, d] and [n_tokens, Hq, n_splits, 2] (unused for one split)

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class KernelLibraryError(RuntimeError):
@@ -32,11 +32,11 @@ _SIGNATURES = {
     "ra_embed": [P, I, P, P, I, I, P],
     "ra_add_rmsnorm": [P, P, P, I, P, I, P, I, I, F, P],
     "ra_qk_norm_rope_cache": [P, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
-    "ra_silu_mul": [P, P, I, I, I, P],
+    "ra_silu_mul": [P, P, I, I, I, I, P],
     "ra_attention_plain": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
-    "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, P],
+    "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
 }

@@ -120,13 +120,18 @@ class HipKernels:
                      int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(),
                      vcache.data_ptr(), kcache.shape[2], T, num_heads, num_kv_heads, head_dim, _stream())
 
-    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0) -> None:
+        """out = silu(gate) * up. ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g
+        gate columns and g up columns alternate."""
         _dev(gate_up, out)
         T, I = out.shape
         if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype \
                 or not gate_up.is_contiguous() or not out.is_contiguous():
             raise ValueError(f"silu_mul: gate_up {tuple(gate_up.shape)} against out {tuple(out.shape)}")
-        library.call("ra_silu_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I, _stream())
+        if group < 0 or (group > 0 and I % group != 0):
+            raise ValueError(f"silu_mul: width {I} is not a whole number of runs of {group}")
+        library.call("ra_silu_mul", gate_up.data_ptr(), out.data_ptr(), _tag(out, "silu_mul"), T, I,
+                     int(group), _stream())
 
     # ------------------------------------------------------------- attention
     SHORT_PORTION = 4     # portions up to this many tokens go token by token through the decode kernel
@@ -318,7 +323,30 @@ class HipKernels:
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
         library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
-                     _tag(out, "linear output"), M, N, K, x.stride(0), out.stride(0), _stream())
+                     _tag(out, "linear output"), 0, M, N, K, x.stride(0), out.stride(0), _stream())
+
+    GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
+
+    def gated_linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+        """out[M, I] = silu(x . Wg^T) * (x . Wu^T) for ``weight`` [2I, K] whose rows alternate in
+        runs of GATE_GROUP: 8 gate rows, the 8 up rows of the same features, and so on.
+
+        bfloat16 with up to 64 rows: one kernel, the gate applied in the product's
+        epilogue. Otherwise the product into a [M, 2I] buffer, then the gate kernel."""
+        _dev(x, weight, out)
+        M, K = x.shape
+        I = out.shape[1]
+        if weight.shape != (2 * I, K) or out.shape != (M, I) or I % self.GATE_GROUP != 0:
+            raise ValueError(f"gated_linear: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 \
+                and M <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1 \
+                and weight.is_contiguous() and out.stride(1) == 1:
+            library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), None, out.data_ptr(),
+                         _tag(out, "linear output"), 1, M, 2 * I, K, x.stride(0), out.stride(0), _stream())
+            return
+        gu = torch.empty((M, 2 * I), dtype=out.dtype, device=x.device)
+        self.linear(x, weight, gu)
+        self.silu_mul(gu, out, self.GATE_GROUP)
 
     # -------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, seeds: torch.Tensor,

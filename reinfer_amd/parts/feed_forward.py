@@ -1,8 +1,11 @@
 """Dense SwiGLU feed-forward: down( silu(gate(x)) * up(x) ), no bias.
 
 crates/cuda/src/engine.rs:4288-4303; silu(g) = g / (1 + exp(-g))
-(crates/cuda/kernels/dense_kernels.cu:202-213). gate and up are one product
-over rows [gate; up], followed by the fused SiLU-gate kernel.
+(crates/cuda/kernels/dense_kernels.cu:202-213). gate and up are one product:
+their rows are interleaved in runs of 8 at load (8 gate rows, the 8 up rows of
+the same features, ...), so that for few tokens the product's epilogue applies
+the gate itself and for many the gate kernel reads both from one cache line.
+A width that is no multiple of 8 keeps [gate; up] and the separate gate kernel.
 """
 from __future__ import annotations
 
@@ -28,18 +31,29 @@ class SwiGLU:
                  dtype: torch.dtype, device: torch.device):
         self.spec = spec
         self.dtype = dtype
-        self.w_gate_up = torch.cat([weights[prefix + "gate_proj.weight"],
-                                    weights[prefix + "up_proj.weight"]], dim=0).contiguous()
+        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        I, h = spec.intermediate, spec.hidden
+        self.group = getattr(kernels.current(), "GATE_GROUP", 0)
+        if self.group and I % self.group == 0:
+            g = self.group
+            self.w_gate_up = torch.stack([gate.view(I // g, g, h), up.view(I // g, g, h)], dim=1) \
+                .reshape(2 * I, h).contiguous()
+        else:
+            self.group = 0
+            self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + "down_proj.weight"]
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         ops = kernels.current()
         T = x.shape[0]
         I = self.spec.intermediate
-        gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
-        ops.linear(x, self.w_gate_up, gu)
         act = torch.empty((T, I), dtype=self.dtype, device=x.device)
-        ops.silu_mul(gu, act)
+        if self.group:
+            ops.gated_linear(x, self.w_gate_up, act)
+        else:
+            gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
+            ops.linear(x, self.w_gate_up, gu)
+            ops.silu_mul(gu, act)
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(act, self.w_down, out)
         return out

@@ -70,10 +70,21 @@ class KernelDouble:
             kcache[s // bs, :, s % bs, :] = k[t].to(kcache.dtype)
             vcache[s // bs, :, s % bs, :] = v[t].to(vcache.dtype)
 
-    def silu_mul(self, gate_up, out):
-        I = out.shape[1]
-        g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
+    GATE_GROUP = 8
+
+    def silu_mul(self, gate_up, out, group=0):
+        T, I = out.shape
+        if group:
+            v = gate_up.view(T, I // group, 2, group).float()
+            g, u = v[:, :, 0].reshape(T, I), v[:, :, 1].reshape(T, I)
+        else:
+            g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
         out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+    def gated_linear(self, x, weight, out):
+        gu = torch.empty((x.shape[0], weight.shape[0]), dtype=out.dtype)
+        self.linear(x, weight, gu)
+        self.silu_mul(gu, out, self.GATE_GROUP)
 
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                   scale, window, group):

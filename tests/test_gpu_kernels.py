@@ -101,6 +101,14 @@ def test_silu_mul(dtype):
     ops().silu_mul(gu, out)
     g, u = gu[:, :I].double(), gu[:, I:].double()
     close(out, g / (1 + torch.exp(-g)) * u, OUT_TOL[dtype])
+    # gate and up interleaved in runs of 3
+    I2 = 330
+    gu2 = gu[:, :2 * I2].contiguous()
+    out2 = torch.empty(T, I2, device=DEV, dtype=DT[dtype])
+    ops().silu_mul(gu2, out2, 3)
+    v = gu2.view(T, I2 // 3, 2, 3).double()
+    g, u = v[:, :, 0].reshape(T, I2), v[:, :, 1].reshape(T, I2)
+    close(out2, g / (1 + torch.exp(-g)) * u, OUT_TOL[dtype])
 
 
 def rope_reference(x, positions, theta, rotary_dim, style):
@@ -384,6 +392,24 @@ def test_linear_skinny(M, N, K, dout):
     ops().linear_skinny(x[M - 1:M], w, one)
     ops().linear_skinny(x, w, out)
     close(one, out[M - 1:M], 1e-6 if dout == "float32" else 2 ** -8)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 20, 33, 64, 65, 200])
+@pytest.mark.parametrize("I,K", [(8, 8), (40, 64), (176, 80), (320, 96), (12288, 512)])
+def test_gated_linear(M, I, K):
+    """silu(x Wg^T) * (x Wu^T) with gate and up rows interleaved in runs of 8: the fused epilogue
+    (up to 64 rows) and the two-kernel form (more rows) against the separate float products."""
+    torch.manual_seed(M + I + K)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    wg = (torch.randn(I, K, device=DEV) * 2 / math.sqrt(K)).to(torch.bfloat16)
+    wu = (torch.randn(I, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    w = torch.stack([wg.view(I // 8, 8, K), wu.view(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
+    out = torch.full((M, I), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().gated_linear(x, w, out)
+    g = x.double() @ wg.double().T
+    u = x.double() @ wu.double().T
+    # the two-kernel form rounds gate and up to bfloat16 before the gate: two more roundings
+    close(out, g / (1 + torch.exp(-g)) * u, 2 ** -8 if M <= 64 else 3 * 2 ** -8)
 
 
 def test_linear_dispatch_refuses_nothing_silently():
