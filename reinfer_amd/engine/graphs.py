@@ -1,0 +1,212 @@
+"""Decode steps as captured HIP graphs.
+
+A step in which every request brings exactly one token has the same shape each
+time; only index arrays change. Such a step is captured once per (padded batch
+size, context bucket) with static input buffers, and later steps copy their
+indices into those buffers (one host-to-device copy) and replay the graph: the
+few hundred launches of a step cost one call. The captured work is the
+product's own forward pass and sampler, run through the same parts and kernels
+as an eager step; nothing is traced or rewritten.
+
+Rows past the step's requests are padding: token 0 at position 0 that stores
+nothing (slot -1, state slot -1) and whose logits nobody reads. A part that keeps
+per-request state and declares itself ``graph_safe`` must leave state slot -1
+alone.
+
+The reference launches every kernel of every step from the host
+(crates/cuda/src/engine.rs:5853-6350) and names graph capture as future work.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import kernels
+from .batch import StepBatch, StepEntry
+
+MAX_GRAPH_BATCH = 64
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class _CapturedStep:
+    """Static buffers and the graph of one (batch size, context bucket)."""
+
+    def __init__(self, runner, B: int, ctx_cap: int, pool):
+        self.runner = runner
+        self.B = B
+        self.ctx_cap = ctx_cap
+        dev = runner.device
+        bs = runner.block_size
+        n_groups = len(runner.manager.groups)
+        W = max(1, -(-runner.max_model_len // bs))
+        self.W = W
+        # layout of the packed int32 buffer (seeds first: they are read as int64)
+        names = [("seeds", 2 * B), ("temps", B), ("sample_pos", B), ("token_ids", B), ("positions", B),
+                 ("seq_of_token", B), ("cu_tokens", B + 1), ("start_pos", B), ("ctx_lens", B),
+                 ("state_slots", B), ("fresh", B), ("logit_rows", B), ("no_slots", B)]
+        for g in range(n_groups):
+            names += [(f"table{g}", B * W), (f"slots{g}", B)]
+        self.off: Dict[str, Tuple[int, int]] = {}
+        o = 0
+        for name, size in names:
+            self.off[name] = (o, o + size)
+            o += size
+        self.host = torch.zeros(o, dtype=torch.int32, pin_memory=True)
+        self.h = self.host.numpy()
+        self.dev = torch.zeros(o, dtype=torch.int32, device=dev)
+
+        def hv(name):
+            a, b = self.off[name]
+            return self.h[a:b]
+
+        def dv(name):
+            a, b = self.off[name]
+            return self.dev[a:b]
+
+        self.h_seeds = hv("seeds").view(np.int64)
+        self.h_temps = hv("temps").view(np.float32)
+        self.h_tables = [hv(f"table{g}").reshape(B, W) for g in range(n_groups)]
+        self.h_slots = [hv(f"slots{g}") for g in range(n_groups)]
+        self._hv = hv
+        # what never changes
+        hv("seq_of_token")[:] = np.arange(B)
+        hv("cu_tokens")[:] = np.arange(B + 1)
+        hv("logit_rows")[:] = np.arange(B)
+        hv("no_slots")[:] = -1
+        self.row_owner: List[Optional[object]] = [None] * B
+        self.row_len = [[0] * B for _ in range(n_groups)]
+        self._pad_rows(0, B)
+
+        self.seeds = dv("seeds").view(torch.int64)
+        self.temps = dv("temps").view(torch.float32)
+        self.sample_pos = dv("sample_pos")
+        self.tokens = torch.zeros(B, dtype=torch.int32, device=dev)
+        self.batch = StepBatch(
+            num_tokens=B, num_seqs=B, num_logit_rows=B,
+            token_ids=dv("token_ids"), positions=dv("positions"), seq_of_token=dv("seq_of_token"),
+            cu_tokens=dv("cu_tokens"), start_pos=dv("start_pos"), ctx_lens=dv("ctx_lens"),
+            state_slots=dv("state_slots"), fresh=dv("fresh"), logit_rows=dv("logit_rows"),
+            no_slots=dv("no_slots"),
+            block_tables=[dv(f"table{g}").view(B, W) for g in range(n_groups)],
+            slots=[dv(f"slots{g}") for g in range(n_groups)],
+            q_lens=[1] * B, starts=[ctx_cap - 1] * B, max_q_len=1, max_ctx_len=ctx_cap)
+        # the kernels choose grids from host-side numbers: fixed for this bucket
+        self.batch.extra["attention_plan"] = {
+            "n_decode": B, "decode_max_ctx": ctx_cap, "decode_list": None, "n_prefill": 0,
+            "prefill_list": None, "n_tiles": 0, "tiles": None}
+        self.logits: Optional[torch.Tensor] = None
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._capture(pool)
+
+    def _pad_rows(self, lo: int, hi: int) -> None:
+        hv = self._hv
+        for name, val in (("token_ids", 0), ("positions", 0), ("start_pos", 0), ("ctx_lens", 1),
+                          ("state_slots", -1), ("fresh", 0), ("sample_pos", 0), ("temps", 0)):
+            hv(name)[lo:hi] = val
+        self.h_seeds[lo:hi] = 0
+        for g, s in enumerate(self.h_slots):
+            s[lo:hi] = -1
+        for i in range(lo, hi):
+            self.row_owner[i] = None
+
+    def _body(self) -> None:
+        r = self.runner
+        self.logits = r.model.forward(self.batch, r.caches)
+        kernels.current().sample(self.logits, self.temps, self.seeds, self.sample_pos, self.tokens)
+
+    def _capture(self, pool) -> None:
+        self.dev.copy_(self.host, non_blocking=True)
+        # once outside the capture: whatever initialises lazily must not be recorded
+        cur = torch.cuda.current_stream()
+        side = torch.cuda.Stream()
+        side.wait_stream(cur)
+        with torch.cuda.stream(side), torch.no_grad():
+            self._body()
+        cur.wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=pool), torch.no_grad():
+            self._body()
+
+    def fill(self, entries: Sequence[StepEntry], rcs, sampling) -> None:
+        bs = self.runner.block_size
+        hv = self._hv
+        tok, pos, start, ctx = hv("token_ids"), hv("positions"), hv("start_pos"), hv("ctx_lens")
+        state, fresh, spos = hv("state_slots"), hv("fresh"), hv("sample_pos")
+        n = len(entries)
+        for i, (e, rc) in enumerate(zip(entries, rcs)):
+            p = rc.num_tokens
+            tok[i] = e.tokens[0]
+            pos[i] = p
+            start[i] = p
+            ctx[i] = p + 1
+            state[i] = rc.slot
+            fresh[i] = 1 if rc.fresh else 0
+            same = self.row_owner[i] is rc
+            for g, table in enumerate(rc.tables):
+                have = self.row_len[g][i] if same else 0
+                if len(table) > have:
+                    # entries given back (-1) are never read; 0 keeps every index valid
+                    self.h_tables[g][i, have:len(table)] = [b if b >= 0 else 0 for b in table[have:]]
+                self.row_len[g][i] = len(table)
+                blk = table[p // bs]
+                self.h_slots[g][i] = -1 if blk < 0 else blk * bs + p % bs
+            self.row_owner[i] = rc
+        if sampling is not None:
+            temps, seeds, positions = sampling
+            self.h_temps[:n] = temps
+            self.h_seeds[:n] = seeds
+            spos[:n] = positions
+        else:
+            self.h_temps[:n] = 0.0
+            self.h_seeds[:n] = 0
+            spos[:n] = 0
+        hi = max(i for i, o in enumerate(self.row_owner) if o is not None) + 1
+        if hi > n:
+            self._pad_rows(n, hi)
+
+    def replay(self) -> None:
+        self.dev.copy_(self.host, non_blocking=True)
+        self.graph.replay()
+
+
+class DecodeGraphs:
+    def __init__(self, runner):
+        self.runner = runner
+        self.steps: Dict[Tuple[int, int], _CapturedStep] = {}
+        self.pool = None
+        self.replays = 0
+
+    def eligible(self, entries: Sequence[StepEntry]) -> bool:
+        if len(entries) > MAX_GRAPH_BATCH:
+            return False
+        return all(len(e.tokens) == 1 for e in entries)
+
+    def run(self, entries: Sequence[StepEntry], sampling=None):
+        """-> (logits [B_pad, vocab] static, tokens [B_pad] static): rows past the
+        entries are padding; both are overwritten by the next replay of this bucket."""
+        r = self.runner
+        rcs = [r.manager.get(e.rid) for e in entries]
+        B = _bucket(len(entries))
+        longest = max(rc.num_tokens for rc in rcs) + 1
+        ctx_cap = max(256, _bucket(longest))
+        ctx_cap = min(ctx_cap, max(256, _bucket(r.max_model_len)))
+        key = (B, ctx_cap)
+        cs = self.steps.get(key)
+        if cs is None:
+            if self.pool is None:
+                self.pool = torch.cuda.graph_pool_handle()
+            cs = _CapturedStep(r, B, ctx_cap, self.pool)
+            self.steps[key] = cs
+        cs.fill(entries, rcs, sampling)
+        cs.replay()
+        self.replays += 1
+        return cs.logits, cs.tokens

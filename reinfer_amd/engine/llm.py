@@ -21,7 +21,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 import torch
 
 from ..config import load_config
-from ..sampling import Sampler, SamplingParams, derive_seed
+from ..sampling import Sampler, SamplingError, SamplingParams, as_int64, derive_seed
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import FINISHED, Request, RequestRefused, Scheduler, StepPlan
@@ -97,16 +97,34 @@ class LLMEngine:
             return finished
         entries, rows = [], []
         for p in plan.portions:
-            toks = p.request.tokens[p.start:p.start + p.length]
-            entries.append(StepEntry(p.request.rid, toks, [p.length - 1] if p.samples else []))
+            r = p.request
+            if p.length == 1:
+                i = p.start
+                toks = [r.prompt[i] if i < len(r.prompt) else r.output[i - len(r.prompt)]]
+            else:
+                toks = r.tokens[p.start:p.start + p.length]
+            entries.append(StepEntry(r.rid, toks, [p.length - 1] if p.samples else []))
             if p.samples:
-                rows.append(p.request)
-        logits = self.runner.step(entries)
+                rows.append(r)
         sampled: Dict[Hashable, int] = {}
-        if rows:
-            toks = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
-                                       [r.num_tokens for r in rows], [r.tokens for r in rows])
-            sampled = {r.rid: t for r, t in zip(rows, toks)}
+        plain = len(rows) == len(entries) and not any(r.params.filters for r in rows)
+        if plain:
+            # every entry wants one token and none shapes its distribution: the step may draw them itself
+            sampling = ([max(0.0, float(r.params.temperature)) for r in rows],
+                        [as_int64(r.seed) for r in rows], [r.num_tokens for r in rows])
+            logits, toks = self.runner.step_sampled(entries, sampling)
+        else:
+            logits, toks = self.runner.step(entries), None
+        if toks is not None:
+            out = toks.tolist()
+            for r, t in zip(rows, out):
+                if t < 0:
+                    raise SamplingError(f"request {r.rid!r}: no finite logit to sample from")
+                sampled[r.rid] = t
+        elif rows:
+            out = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
+                                      [r.num_tokens for r in rows], [r.tokens for r in rows])
+            sampled = {r.rid: t for r, t in zip(rows, out)}
         done = self.scheduler.complete(plan, sampled)
         return finished + [self._output(r) for r in done]
 

@@ -44,7 +44,8 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
                  device: torch.device, *, block_size: int = 16, num_blocks: Optional[int] = None,
                  max_tokens: Optional[int] = None, max_seqs: int = 64,
-                 max_model_len: Optional[int] = None, memory_fraction: float = 0.9):
+                 max_model_len: Optional[int] = None, memory_fraction: float = 0.9,
+                 use_graphs: Optional[bool] = None):
         self.spec = spec
         self.dtype = dtype
         self.device = device
@@ -96,6 +97,16 @@ class ModelRunner:
                 self.caches.append(LayerCache(state=state))
             else:
                 self.caches.append(None)
+
+        # decode steps replay captured graphs when every part says it can be captured
+        safe = all(getattr(getattr(b, "mixer", None), "graph_safe", False)
+                   and getattr(getattr(b, "ffn", None), "graph_safe", False) for b in self.model.blocks)
+        if use_graphs is None:
+            use_graphs = True
+        self.graphs = None
+        if use_graphs and safe and device.type == "cuda":
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self)
 
     # ------------------------------------------------------------ building
     @classmethod
@@ -182,7 +193,15 @@ class ModelRunner:
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the entries' tokens as one batch; logits [wanted, vocab] float32,
-        in the order of the entries and of each entry's ``want``."""
+        in the order of the entries and of each entry's ``want``. The result may be
+        a view of a buffer that the next step overwrites: use it before stepping again."""
+        return self.step_sampled(entries, None)[0]
+
+    def step_sampled(self, entries: Sequence[StepEntry], sampling=None):
+        """As :meth:`step`; ``sampling`` = (temperatures, seeds, positions), one per entry,
+        asks for a token from each entry's single wanted row where the step can draw it
+        itself. -> (logits, tokens): ``tokens`` is an int32 device tensor, one per
+        entry, or None when the caller has to sample from the logits."""
         self.check_entries(entries)
         growth = [(e.rid, self.manager.get(e.rid).num_tokens + len(e.tokens)) for e in entries]
         if not self.manager.can_grow(growth):
@@ -192,11 +211,24 @@ class ModelRunner:
             raise OutOfBlocks(g, need[g], self.manager.pools[g].num_free)
         for rid, total in growth:
             self.manager.grow(rid, total)
-        batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
-        logits = self.forward(batch)
+        tokens = None
+        if self.graphs is not None and self.graphs.eligible(entries):
+            all_logits, all_tokens = self.graphs.run(entries, sampling)
+            n = len(entries)
+            if all(len(e.want) == 1 for e in entries):
+                logits = all_logits[:n]
+                if sampling is not None:
+                    tokens = all_tokens[:n]
+            else:
+                rows = [i for i, e in enumerate(entries) for _ in e.want]
+                logits = all_logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows \
+                    else all_logits[:0]
+        else:
+            batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
+            logits = self.forward(batch)
         for rid, total in growth:
             self.manager.commit(rid, total)
-        return logits
+        return logits, tokens
 
     def forward(self, batch: StepBatch) -> torch.Tensor:
         with torch.no_grad():

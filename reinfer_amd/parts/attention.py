@@ -23,6 +23,8 @@ from .registry import lookup, register_mixer
 
 @register_mixer("gqa_attention")
 class GroupedQueryAttention:
+    graph_safe = True       # no host-side state: a decode step with it can be captured
+
     @classmethod
     def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
         nq = spec.num_heads * spec.head_dim

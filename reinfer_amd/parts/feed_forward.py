@@ -21,6 +21,8 @@ from .registry import register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU:
+    graph_safe = True       # no host-side state: a decode step with it can be captured
+
     @classmethod
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
         return [ParamDecl(prefix + "gate_proj.weight", (spec.intermediate, spec.hidden)),

@@ -1,4 +1,4 @@
 from .params import SamplingParams
-from .sampler import Sampler, SamplingError, derive_seed
+from .sampler import Sampler, SamplingError, as_int64, derive_seed
 
-__all__ = ["SamplingParams", "Sampler", "SamplingError", "derive_seed"]
+__all__ = ["SamplingParams", "Sampler", "SamplingError", "as_int64", "derive_seed"]

@@ -33,7 +33,7 @@ def derive_seed(engine_seed: int, arrival: int) -> int:
     return splitmix64((engine_seed ^ arrival) & ((1 << 64) - 1))
 
 
-def _as_int64(seed: int) -> int:
+def as_int64(seed: int) -> int:
     seed &= (1 << 64) - 1
     return seed - (1 << 64) if seed >= (1 << 63) else seed
 
@@ -56,7 +56,7 @@ class Sampler:
             logits = logits.clone()
             ops.filter_logits(logits, params, histories)
         temp = torch.tensor([max(0.0, float(p.temperature)) for p in params], dtype=torch.float32)
-        seeds_t = torch.tensor([_as_int64(int(s)) for s in seeds], dtype=torch.int64)
+        seeds_t = torch.tensor([as_int64(int(s)) for s in seeds], dtype=torch.int64)
         pos_t = torch.tensor([int(p) for p in positions], dtype=torch.int32)
         tokens = torch.empty(n, dtype=torch.int32, device=self.device)
         ops.sample(logits, temp.to(self.device), seeds_t.to(self.device), pos_t.to(self.device), tokens)
