@@ -79,15 +79,92 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
   }
 }
 
+// The same for rows that fit the workgroup's registers (width a multiple of 4, at
+// most threads * 16): one read of the row, the sum in registers, one write. A
+// decode step runs this on a handful of rows, so its time is the chain of memory
+// round trips, not bandwidth; the plain kernel above reads the row a second time.
+typedef float f32x4_raw __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ f32x4_raw load(const float* p) { return *(const f32x4_raw*)p; }
+  static __device__ __forceinline__ void store(float* p, f32x4_raw v) { *(f32x4_raw*)p = v; }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ f32x4_raw load(const bf16_t* p) {
+    const bf16x4_t v = *(const bf16x4_t*)p;
+    return (f32x4_raw){(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, f32x4_raw v) {
+    *(bf16x4_t*)p = (bf16x4_t){(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+  }
+};
+
+#define NORM_CH 4       // chunks of 4 elements a thread keeps
+
+template <typename TA, typename TW>
+__global__ void add_rmsnorm_reg_kernel(float* __restrict__ resid, const TA* __restrict__ delta,
+                                       const TW* __restrict__ w, TA* __restrict__ out,
+                                       const int* __restrict__ rows, int h, float eps) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* x = resid + src * h;
+  const TA* dl = delta ? delta + src * h : nullptr;
+  f32x4_raw v[NORM_CH], wv[NORM_CH];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NORM_CH; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    v[j] = (f32x4_raw){0.f, 0.f, 0.f, 0.f};
+    wv[j] = v[j];
+    if (i < h) {
+      v[j] = Vec4<float>::load(x + i);
+      if (dl) v[j] += Vec4<TA>::load(dl + i);
+      wv[j] = Vec4<TW>::load(w + i);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NORM_CH; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    if (i < h) {
+      if (dl && !rows) Vec4<float>::store(x + i, v[j]);
+      ss += v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss / (float)h + eps);
+  TA* o = out + (size_t)r * h;
+#pragma unroll
+  for (int j = 0; j < NORM_CH; ++j) {
+    const int i = (threadIdx.x + j * blockDim.x) * 4;
+    if (i < h) Vec4<TA>::store(o + i, v[j] * rstd * wv[j]);
+  }
+}
+
 extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weight, int weight_dtype,
                               void* out, int act_dtype, const int* rows, int n_rows, int hidden,
                               float eps, hipStream_t stream) {
   RA_CHECK(n_rows > 0 && hidden > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_rows, hidden);
-  const int threads = hidden >= 2048 ? 512 : 256;
-#define RA_GO(TA, TW)                                                                           \
-  add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta,          \
-                                                             (const TW*)weight, (TA*)out, rows, \
-                                                             hidden, eps)
+  int threads = hidden >= 2048 ? 512 : 256;
+  const bool aligned = hidden % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                       ((uintptr_t)weight % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+  bool in_regs = aligned && hidden <= 1024 * 4 * NORM_CH;
+  if (in_regs) {
+    threads = 64;
+    while (threads * 4 * NORM_CH < hidden) threads *= 2;
+    if (hidden >= 2048 && threads < 256) threads = 256;
+  }
+#define RA_GO(TA, TW)                                                                                  \
+  do {                                                                                                 \
+    if (in_regs)                                                                                       \
+      add_rmsnorm_reg_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(                                  \
+          resid, (const TA*)delta, (const TW*)weight, (TA*)out, rows, hidden, eps);                    \
+    else                                                                                               \
+      add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, stream>>>(resid, (const TA*)delta,             \
+                                                                 (const TW*)weight, (TA*)out, rows,    \
+                                                                 hidden, eps);                         \
+  } while (0)
   if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GO(float, float);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GO(bf16_t, bf16_t);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GO(bf16_t, float);

@@ -64,7 +64,7 @@ def test_embed(dtype):
 
 
 @pytest.mark.parametrize("dtype,wdtype", [("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")])
-@pytest.mark.parametrize("h", [100, 4104])
+@pytest.mark.parametrize("h", [100, 98, 4096, 4104, 20000])
 def test_add_rmsnorm(dtype, wdtype, h):
     torch.manual_seed(h)
     T, eps = 7, 1e-5
