@@ -1,15 +1,26 @@
-// Flash-decode attention over the paged cache, bfloat16: one query token per
-// (request, position), the query heads of one KV head handled together so that
-// every key and value is read once for the whole group, the keys split over
-// several workgroups (split-KV) and merged by a second small kernel.
+// Flash-decode attention over the paged cache, bfloat16, on the matrix cores:
+// one query token per (request, position); the query heads of one KV head are
+// the columns of the MFMA tiles, so every key and value is read once for the
+// whole group. The keys are cut into chunks; a workgroup (4 waves) takes one
+// (chunk, KV head, token), its waves take 32 keys at a time:
 //
-// A workgroup of 256 threads takes (split, KV head, token). A key's row of d
-// elements is spread over d/8 adjacent lanes, 16 bytes a lane, so a wavefront
-// reads whole rows, consecutive keys of a block back to back. Each group of
-// lanes keeps its own running maximum, sum and weighted values (online
-// softmax, float), so the key loop has no workgroup barrier; the groups are
-// merged once at the end (shuffles inside a wavefront, LDS across wavefronts).
-// Dot products use v_dot2_f32_bf16 (float accumulate).
+//   S^T[key][head]  = K . Q^T          v_mfma_f32_16x16x32_bf16 over d
+//   online softmax per head column     (float: running maximum and sum)
+//   O^T[d][head]   += V^T . P          contraction over the 32 keys
+//
+// The cache keeps K and V in tiles of 16 slots laid out in MFMA operand order
+// (cache_k_index / cache_v_index), so a wave's load of an operand is one
+// contiguous run of 1 KB (K) or 512 bytes (V^T) and goes straight from memory
+// into the matrix core's registers; the probabilities are the second
+// product's operand as they leave the first (k-slot s of lane group g is key
+// 4g + s of the first 16 keys for s < 4, of the second 16 for s >= 4, for both
+// operands alike).
+//
+// Chunks of one (token, head) are merged by a second small kernel, always in
+// chunk order. (Merging in the last workgroup to arrive needs device-wide
+// release/acquire fences in every workgroup; on this chip each one writes back
+// and invalidates a whole L2, which made the kernel seven times slower.) A token
+// whose keys fit one chunk is written directly.
 //
 // The reference's flash decode keeps the whole score row in shared memory,
 // which caps the context at (d + max_kv) * 4 <= 48 KB (crates/cuda/src/decode.rs:49-52;
@@ -19,271 +30,297 @@
 #include "reinfer_hip.h"
 
 #define FD_THREADS 256
-#define FD_U 4
+#define FD_WAVES 4
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// DLP: lanes per key row (a power of two >= d/8); G: query heads per KV head
-template <int DLP, int G>
+template <int DMAX>
 __global__ void __launch_bounds__(FD_THREADS)
 flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                     const int* __restrict__ block_tables, int max_blocks,
                     const int* __restrict__ token_list, const int* __restrict__ seq_of_token,
-                    const int* __restrict__ positions, int block_size, int Hkv, int d,
-                    float scale_log2, int window, int n_splits, float* __restrict__ part_o,
-                    float* __restrict__ part_ml) {
-  constexpr int NSUB = FD_THREADS / DLP;          // key rows a workgroup reads per load
-  constexpr int SUB_PER_WAVE = RA_WAVE / DLP;
-  __shared__ float lds_o[FD_THREADS / RA_WAVE][G][DLP * 8];
-  __shared__ float lds_ml[FD_THREADS / RA_WAVE][G][2];
+                    const int* __restrict__ positions, int block_size, int Hkv, int G, int d,
+                    float scale_log2, int window, int chunk, int max_chunks,
+                    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
+  constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
+  extern __shared__ float lds[];       // [waves][G][d] outputs, then [waves][G][2] maximum and sum
 
-  const int split = blockIdx.x, kvh = blockIdx.y, li = blockIdx.z;
+  const int ci = blockIdx.x, kvh = blockIdx.y, li = blockIdx.z;
   const int t = token_list ? token_list[li] : li;
-  const int seq = seq_of_token[t];
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int n_keys = p + 1 - lo;
-  int chunk = (n_keys + n_splits - 1) / n_splits;
-  chunk = (chunk + NSUB * FD_U - 1) / (NSUB * FD_U) * (NSUB * FD_U);
-  const int start = lo + split * chunk;
-  const int end = min(p + 1, start + chunk);
-
-  const int tid = threadIdx.x;
-  const int dc = tid % DLP, sub = tid / DLP;
-  const int DL = d / 8;
-  const bool active = dc < DL;
-  const int Hq = Hkv * G;
+  const int c_first = lo / chunk, c_last = p / chunk;
+  if (ci < c_first || ci > c_last) return;       // no key of this token in the chunk
+  const int n_chunks = c_last - c_first + 1;
+  const int seq = seq_of_token[t];
   const int* table = block_tables + (size_t)seq * max_blocks;
 
-  // this lane's 8 elements of each query head of the group, as bfloat16 pairs
-  bf16x2_t qp[G][4];
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (active) v = *(const bf16x8_t*)(q + (size_t)t * q_stride + (size_t)(kvh * G + h) * d + dc * 8);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) qp[h][j] = (bf16x2_t){v[2 * j], v[2 * j + 1]};
-  }
-  float m[G], l[G], acc[G][8];
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    m[h] = -INFINITY;
-    l[h] = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
-  }
+  const int tid = threadIdx.x;
+  const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  const int Hq = Hkv * G;
 
-  for (int base = start; base < end; base += NSUB * FD_U) {
-    bf16x8_t kx[FD_U], vx[FD_U];
-    bool ok[FD_U];
+  // second operand of the score product: column r is query head r of the group
+  bf16x8_t qreg[NDT];
 #pragma unroll
-    for (int u = 0; u < FD_U; ++u) {
-      const int key = base + u * NSUB + sub;
-      ok[u] = key < end;
-      kx[u] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
-      vx[u] = kx[u];
-      if (ok[u] && active) {
-        const int blk = table[key / block_size];
-        const size_t off = (((size_t)blk * Hkv + kvh) * block_size + key % block_size) * d + dc * 8;
-        kx[u] = *(const bf16x8_t*)(kcache + off);
-        vx[u] = *(const bf16x8_t*)(vcache + off);
-      }
-    }
-    float s[FD_U][G];
-#pragma unroll
-    for (int u = 0; u < FD_U; ++u) {
-#pragma unroll
-      for (int h = 0; h < G; ++h) {
-        float dot = 0.f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          dot = __builtin_amdgcn_fdot2_f32_bf16((bf16x2_t){kx[u][2 * j], kx[u][2 * j + 1]}, qp[h][j], dot, false);
-#pragma unroll
-        for (int o = DLP / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, RA_WAVE);
-        s[u][h] = ok[u] ? dot * scale_log2 : -INFINITY;
-      }
-    }
-    float vf[FD_U][8];
-#pragma unroll
-    for (int u = 0; u < FD_U; ++u)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) vf[u][j] = (float)vx[u][j];
-#pragma unroll
-    for (int h = 0; h < G; ++h) {
-      float mn = m[h];
-#pragma unroll
-      for (int u = 0; u < FD_U; ++u) mn = fmaxf(mn, s[u][h]);
-      if (mn == -INFINITY) continue;           // nothing seen yet and nothing here
-      const float corr = fast_exp2(m[h] - mn);  // m = -inf gives 0
-      float pr[FD_U], psum = 0.f;
-#pragma unroll
-      for (int u = 0; u < FD_U; ++u) {
-        pr[u] = fast_exp2(s[u][h] - mn);        // masked keys: exp2(-inf) = 0
-        psum += pr[u];
-      }
-      l[h] = l[h] * corr + psum;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float a = acc[h][j] * corr;
-#pragma unroll
-        for (int u = 0; u < FD_U; ++u) a = fmaf(pr[u], vf[u][j], a);
-        acc[h][j] = a;
-      }
-      m[h] = mn;
-    }
+  for (int dt = 0; dt < NDT; ++dt) {
+    const int e = dt * 32 + g * 8;
+    qreg[dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+    if (r < G && e < d) qreg[dt] = *(const bf16x8_t*)(q + (size_t)t * q_stride + (size_t)(kvh * G + r) * d + e);
   }
+  f32x4_t acc[NOT];
+#pragma unroll
+  for (int i = 0; i < NOT; ++i) acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
 
-  // merge the lane groups of a wavefront (same d chunk, different keys)
+  const int k_begin = ci * chunk;
+  const int k_end = min(k_begin + chunk, p + 1);
+  for (int k0 = k_begin + wave * 32; k0 < k_end; k0 += FD_WAVES * 32) {
+    if (k0 + 31 < lo) continue;
+    // the two 16-key tiles of this step; a tile past the last key is not touched
+    bool live[2], edge[2];
+    const bf16_t* kb[2];
+    const bf16_t* vb[2];
 #pragma unroll
-  for (int o = DLP; o < RA_WAVE; o <<= 1) {
+    for (int tt = 0; tt < 2; ++tt) {
+      const int kt = k0 + tt * 16;
+      live[tt] = kt <= p && kt + 15 >= lo;
+      edge[tt] = kt + 15 > p || kt < lo;
+      const int blk = live[tt] ? table[kt / block_size] : 0;
+      const size_t tile = ((size_t)blk * Hkv + kvh) * block_size * d + (size_t)((kt % block_size) >> 4) * 16 * d;
+      kb[tt] = kcache + tile + (g * 16 + r) * 8;        // chunk 4 dt + g of slot r
+      vb[tt] = vcache + tile + (g * 16 + r) * 4;        // slots 4g..4g+3 of row 16 ot + r
+    }
+    bf16x8_t kreg[2][NDT];
+    bf16x4_t vreg[2][NOT];
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      const float mo = __shfl_xor(m[h], o, RA_WAVE);
-      const float mn = fmaxf(m[h], mo);
-      const float c = (mn == -INFINITY) ? 0.f : fast_exp2(m[h] - mn);
-      const float ls = l[h] * c;
-      l[h] = ls + __shfl_xor(ls, o, RA_WAVE);
+    for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float a = acc[h][j] * c;
-        acc[h][j] = a + __shfl_xor(a, o, RA_WAVE);
+      for (int dt = 0; dt < NDT; ++dt) {
+        kreg[tt][dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+        if (live[tt] && dt * 32 + g * 8 < d) kreg[tt][dt] = *(const bf16x8_t*)(kb[tt] + dt * 512);
       }
-      m[h] = mn;
+#pragma unroll
+      for (int ot = 0; ot < NOT; ++ot) {
+        vreg[tt][ot] = (bf16x4_t){0, 0, 0, 0};
+        if (live[tt] && ot * 16 < d) vreg[tt][ot] = *(const bf16x4_t*)(vb[tt] + ot * 256);
+      }
+    }
+    f32x4_t s[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        if (dt * 32 < d) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[tt][dt], qreg[dt], s[tt], 0, 0, 0);
+    }
+    // mask and scale; keys outside [lo, p] get -inf, whatever bits their slots hold
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + tt * 16 + 4 * g + i;
+        const float v = (key <= p && key >= lo) ? s[tt][i] * scale_log2 : -INFINITY;
+        s[tt][i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
+    const float mn = fmaxf(m, tmax);              // finite: the step holds at least one visible key
+    const float corr = fd_exp2(m - mn);           // m = -inf gives 0
+    bf16x8_t pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = fd_exp2(s[tt][i] - mn);  // masked: exp2(-inf) = 0
+        psum += pr;
+        pb[tt * 4 + i] = from_f32<bf16_t>(pr);
+      }
+    l = l * corr + psum;
+    m = mn;
+    // values of masked keys may be anything (a freed block's bits): zero them at the edges
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+      if (edge[tt]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + tt * 16 + 4 * g + i;
+          if (!(key <= p && key >= lo)) {
+#pragma unroll
+            for (int ot = 0; ot < NOT; ++ot) vreg[tt][ot][i] = (bf16_t)0.f;
+          }
+        }
+      }
+#pragma unroll
+    for (int ot = 0; ot < NOT; ++ot) {
+      if (ot * 16 < d) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[ot][i] *= corr;
+        const bf16x8_t a = {vreg[0][ot][0], vreg[0][ot][1], vreg[0][ot][2], vreg[0][ot][3],
+                            vreg[1][ot][0], vreg[1][ot][1], vreg[1][ot][2], vreg[1][ot][3]};
+        acc[ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[ot], 0, 0, 0);
+      }
     }
   }
-  // across wavefronts through LDS
-  const int wave = tid / RA_WAVE, lane = tid % RA_WAVE;
-  if (lane < DLP) {
+  // lane groups hold partial sums of l over their own keys
+  l += __shfl_xor(l, 16, RA_WAVE);
+  l += __shfl_xor(l, 32, RA_WAVE);
+
+  // merge the waves through LDS: lane (head r, group g) holds O^T rows 16 ot + 4 g + i
+  float* lds_o = lds;                                  // [waves][G][d]
+  float* lds_ml = lds + FD_WAVES * G * d;              // [waves][G][2]
+  if (r < G) {
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
+    for (int ot = 0; ot < NOT; ++ot)
+      if (ot * 16 < d) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) lds_o[wave][h][lane * 8 + j] = acc[h][j];
-      if (lane == 0) {
-        lds_ml[wave][h][0] = m[h];
-        lds_ml[wave][h][1] = l[h];
+        for (int i = 0; i < 4; ++i) lds_o[((size_t)wave * G + r) * d + ot * 16 + 4 * g + i] = acc[ot][i];
       }
+    if (g == 0) {
+      lds_ml[(wave * G + r) * 2] = m;
+      lds_ml[(wave * G + r) * 2 + 1] = l;
     }
   }
   __syncthreads();
-  constexpr int NW = FD_THREADS / RA_WAVE;
-  for (int idx = tid; idx < G * DL * 8; idx += FD_THREADS) {
-    const int h = idx / (DL * 8), e = idx % (DL * 8);
-    float mn = -INFINITY;
+  const size_t pair = (size_t)li * Hkv + kvh;
+  const size_t prow = (pair * max_chunks + (ci - c_first)) * G;      // [pair][chunk][head]
+  for (int idx = tid; idx < G * d; idx += FD_THREADS) {
+    const int h = idx / d, e = idx % d;
+    float mw = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) mn = fmaxf(mn, lds_ml[w][h][0]);
+    for (int w = 0; w < FD_WAVES; ++w) mw = fmaxf(mw, lds_ml[(w * G + h) * 2]);
     float lt = 0.f, ot = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const float c = (mn == -INFINITY) ? 0.f : fast_exp2(lds_ml[w][h][0] - mn);
-      lt += lds_ml[w][h][1] * c;
-      ot += lds_o[w][h][e] * c;
+    for (int w = 0; w < FD_WAVES; ++w) {
+      const float mwv = lds_ml[(w * G + h) * 2];
+      const float c = (mwv == -INFINITY) ? 0.f : fd_exp2(mwv - mw);
+      lt += lds_ml[(w * G + h) * 2 + 1] * c;
+      ot += lds_o[((size_t)w * G + h) * d + e] * c;
     }
-    const int head = kvh * G + h;
-    if (n_splits == 1) {
-      out[(size_t)t * out_stride + (size_t)head * d + e] = from_f32<bf16_t>(ot / lt);
+    if (n_chunks == 1) {
+      out[(size_t)t * out_stride + (size_t)(kvh * G + h) * d + e] = from_f32<bf16_t>(ot / lt);
     } else {
-      const size_t row = ((size_t)li * Hq + head) * n_splits + split;
-      part_o[row * d + e] = ot;
+      part_o[(prow + h) * d + e] = ot;
       if (e == 0) {
-        part_ml[row * 2] = mn;
-        part_ml[row * 2 + 1] = lt;
+        part_ml[(prow + h) * 2] = mw;
+        part_ml[(prow + h) * 2 + 1] = lt;
       }
     }
   }
 }
 
-// merge the splits of one (token, head): fixed order, float
-__global__ void flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                          bf16_t* __restrict__ out, int out_stride,
-                                          const int* __restrict__ token_list, int Hq, int d, int n_splits) {
+// Merge of the chunks of one (token, head), one wave each: lane c weighs chunk c
+// (all maxima and sums are read at once), then the lanes share the d outputs.
+__global__ void __launch_bounds__(RA_WAVE)
+flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                          bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
+                          const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk,
+                          int max_chunks) {
   const int head = blockIdx.x, li = blockIdx.y;
   const int t = token_list ? token_list[li] : li;
-  const size_t row0 = ((size_t)li * Hq + head) * n_splits;
-  float mn = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mn = fmaxf(mn, part_ml[(row0 + s) * 2]);
-  float lt = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = part_ml[(row0 + s) * 2];
-    lt += (ms == -INFINITY) ? 0.f : part_ml[(row0 + s) * 2 + 1] * fast_exp2(ms - mn);
-  }
-  for (int e = threadIdx.x; e < d; e += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = part_ml[(row0 + s) * 2];
-      if (ms != -INFINITY) o += part_o[(row0 + s) * d + e] * fast_exp2(ms - mn);
+  const int p = positions[t];
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int n_chunks = p / chunk - lo / chunk + 1;
+  if (n_chunks == 1) return;                           // written by the first kernel
+  const int lane = threadIdx.x;
+  const int kvh = head / G, h = head % G;
+  const size_t base = ((size_t)li * Hkv + kvh) * max_chunks * G + h;    // row of chunk 0; chunks are G rows apart
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};                 // d <= 256: up to 4 outputs a lane
+  float mt = -INFINITY, lt = 0.f;
+  for (int c0 = 0; c0 < n_chunks; c0 += RA_WAVE) {
+    const int c = c0 + lane;
+    float mc = -INFINITY, lc = 0.f;
+    if (c < n_chunks) {
+      mc = part_ml[(base + (size_t)c * G) * 2];
+      lc = part_ml[(base + (size_t)c * G) * 2 + 1];
     }
-    out[(size_t)t * out_stride + (size_t)head * d + e] = from_f32<bf16_t>(o / lt);
+    const float mn = fmaxf(mt, wave_max(mc));          // finite: every chunk saw at least one key
+    const float corr = fd_exp2(mt - mn);
+    const float w = (c < n_chunks) ? fd_exp2(mc - mn) : 0.f;
+    lt = lt * corr + wave_sum(lc * w);
+    mt = mn;
+    const int n_here = min(RA_WAVE, n_chunks - c0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= corr;
+    // four chunks' rows are requested before the first is used
+    for (int cc = 0; cc < n_here; cc += 4) {
+      float v[4][4], wc[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool ok = cc + u < n_here;
+        wc[u] = ok ? __shfl(w, cc + u, RA_WAVE) : 0.f;
+        const float* po = part_o + (base + (size_t)(c0 + (ok ? cc + u : cc)) * G) * d;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e = lane + i * RA_WAVE;
+          v[u][i] = (e < d) ? po[e] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += v[u][i] * wc[u];
+    }
   }
-}
-
-template <int DLP>
-static int launch_fd(int G, dim3 grid, hipStream_t stream, const bf16_t* q, int q_stride, bf16_t* out,
-                     int out_stride, const bf16_t* kc, const bf16_t* vc, const int* tables, int max_blocks,
-                     const int* token_list, const int* seq_of_token, const int* positions, int block_size,
-                     int Hkv, int d, float scale_log2, int window, int n_splits, float* part_o,
-                     float* part_ml) {
-#define RA_FD(GG)                                                                                    \
-  case GG:                                                                                           \
-    flash_decode_kernel<DLP, GG><<<grid, FD_THREADS, 0, stream>>>(                                   \
-        q, q_stride, out, out_stride, kc, vc, tables, max_blocks, token_list, seq_of_token,          \
-        positions, block_size, Hkv, d, scale_log2, window, n_splits, part_o, part_ml);               \
-    break;
-  switch (G) {
-    RA_FD(1) RA_FD(2) RA_FD(3) RA_FD(4) RA_FD(5) RA_FD(6) RA_FD(7) RA_FD(8)
-    default:
-      return ra_fail("attention_decode: %d query heads per KV head (this kernel takes 1..8)", G);
+  const float inv = 1.f / lt;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = lane + i * RA_WAVE;
+    if (e < d) out[(size_t)t * out_stride + (size_t)head * d + e] = from_f32<bf16_t>(acc[i] * inv);
   }
-#undef RA_FD
-  RA_LAUNCH_CHECK("attention_decode");
-  return 0;
 }
 
 // 1 if the kernel takes these sizes, else 0 (the caller then uses the plain kernel)
-extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d) {
+extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return 0;
   const int G = Hq / Hkv;
-  return (G >= 1 && G <= 8 && d % 8 == 0 && d >= 16 && d <= 256) ? 1 : 0;
+  return (G >= 1 && G <= 16 && d % 16 == 0 && d >= 16 && d <= 256 && block_size > 0 &&
+          block_size % 16 == 0) ? 1 : 0;
 }
 
 extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride,
                                    const void* kcache, const void* vcache, const int* block_tables,
                                    int max_blocks, const int* token_list, const int* seq_of_token,
                                    const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
-                                   int d, float scale, int window, int n_splits, float* part_o,
-                                   float* part_ml, hipStream_t stream) {
+                                   int d, float scale, int window, int chunk, int max_chunks,
+                                   float* part_o, float* part_ml, hipStream_t stream) {
   RA_CHECK(n_tokens > 0, "attention_decode: no tokens");
-  RA_CHECK(ra_attention_decode_supports(Hq, Hkv, d),
-           "attention_decode: unsupported sizes (%d query heads, %d KV heads, head size %d)", Hq, Hkv, d);
-  RA_CHECK(block_size > 0 && max_blocks > 0 && window >= 0, "attention_decode: bad cache geometry");
-  RA_CHECK(n_splits >= 1 && n_splits <= 256, "attention_decode: %d splits outside 1..256", n_splits);
-  RA_CHECK(n_splits == 1 || (part_o && part_ml), "attention_decode: split-KV needs the partial buffers");
+  RA_CHECK(ra_attention_decode_supports(Hq, Hkv, d, block_size),
+           "attention_decode: unsupported sizes (%d query heads, %d KV heads, head size %d, block %d)", Hq,
+           Hkv, d, block_size);
+  RA_CHECK(max_blocks > 0 && window >= 0, "attention_decode: bad cache geometry");
+  RA_CHECK(chunk >= 128 && chunk % 128 == 0, "attention_decode: chunk %d is no multiple of 128", chunk);
+  RA_CHECK(max_chunks >= 1 && max_chunks <= 65535, "attention_decode: %d chunks outside 1..65535", max_chunks);
+  RA_CHECK(max_chunks == 1 || (part_o && part_ml),
+           "attention_decode: more than one chunk needs the partial buffers");
   RA_CHECK(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                ((uintptr_t)vcache % 16) == 0,
            "attention_decode: operands must be 16-byte aligned");
   RA_CHECK(n_tokens <= 65535 && Hkv <= 65535, "attention_decode: grid too large");
   const int G = Hq / Hkv;
-  const int DL = d / 8;
-  dim3 grid(n_splits, Hkv, n_tokens);
+  dim3 grid(max_chunks, Hkv, n_tokens);
   const float scale_log2 = scale * 1.4426950408889634f;
-  int rc;
-#define RA_ARGS                                                                                       \
-  G, grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,      \
-      (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions,          \
-      block_size, Hkv, d, scale_log2, window, n_splits, part_o, part_ml
-  if (DL <= 2) rc = launch_fd<2>(RA_ARGS);
-  else if (DL <= 4) rc = launch_fd<4>(RA_ARGS);
-  else if (DL <= 8) rc = launch_fd<8>(RA_ARGS);
-  else if (DL <= 16) rc = launch_fd<16>(RA_ARGS);
-  else rc = launch_fd<32>(RA_ARGS);
-#undef RA_ARGS
-  if (rc) return rc;
-  if (n_splits > 1) {
+  const size_t lds = (size_t)FD_WAVES * G * (d + 2) * sizeof(float);
+  RA_CHECK(lds <= 64 * 1024, "attention_decode: %d heads of %d per KV head need too much LDS", G, d);
+#define RA_FD(DM)                                                                                     \
+  flash_decode_kernel<DM><<<grid, FD_THREADS, lds, stream>>>(                                         \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
+      (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions,           \
+      block_size, Hkv, G, d, scale_log2, window, chunk, max_chunks, part_o, part_ml)
+  if (d <= 64) RA_FD(64);
+  else if (d <= 128) RA_FD(128);
+  else RA_FD(256);
+#undef RA_FD
+  RA_LAUNCH_CHECK("attention_decode");
+  if (max_chunks > 1) {
     dim3 mg(Hq, n_tokens);
-    flash_decode_merge_kernel<<<mg, 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride,
-                                                     token_list, Hq, d, n_splits);
+    flash_decode_merge_kernel<<<mg, RA_WAVE, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, token_list,
+                                                         positions, Hkv, G, d, window, chunk, max_chunks);
     RA_LAUNCH_CHECK("attention_decode merge");
   }
   return 0;

@@ -47,9 +47,10 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
     float s = -INFINITY;
     if (key <= p) {
       const int blk = table[key / block_size];
-      const TA* kr = kcache + (((size_t)blk * Hkv + kvh) * block_size + key % block_size) * d;
+      const TA* kr = kcache + ((size_t)blk * Hkv + kvh) * block_size * d;
+      const int off = key % block_size;
       float dot = 0.f;
-      for (int i = 0; i < d; ++i) dot += qs[i] * to_f32(kr[i]);
+      for (int i = 0; i < d; ++i) dot += qs[i] * to_f32(kr[cache_k_index(off, i, d)]);
       s = dot * scale;
     }
     const float cmax = wave_max(s);
@@ -71,8 +72,8 @@ __global__ void attention_plain_kernel(const TA* __restrict__ q, int q_stride, T
           for (int kk = 0; kk < n_keys; ++kk) {
             const int key2 = base + kk;
             const int blk = table[key2 / block_size];
-            const TA* vr = vcache + (((size_t)blk * Hkv + kvh) * block_size + key2 % block_size) * d;
-            sum += ps[kk] * to_f32(vr[i]);
+            const TA* vr = vcache + ((size_t)blk * Hkv + kvh) * block_size * d;
+            sum += ps[kk] * to_f32(vr[cache_v_index(key2 % block_size, i, d)]);
           }
         }
         acc[r] = acc[r] * corr + sum;
@@ -98,7 +99,9 @@ extern "C" int ra_attention_plain(const void* q, int q_stride, void* out, int ou
   RA_CHECK(n_tokens > 0, "attention_plain: no tokens");
   RA_CHECK(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "attention_plain: %d query heads do not divide into %d groups", Hq, Hkv);
   RA_CHECK(d > 0 && d <= 512, "attention_plain: head size %d outside 1..512", d);
-  RA_CHECK(block_size > 0 && max_blocks > 0, "attention_plain: bad cache geometry");
+  RA_CHECK(block_size > 0 && block_size % 16 == 0 && d % 16 == 0 && max_blocks > 0,
+           "attention_plain: the cache is tiled 16 x 16: block size %d and head size %d must be multiples of 16",
+           block_size, d);
   RA_CHECK(window >= 0, "attention_plain: negative window");
   RA_CHECK(n_tokens <= 65535, "attention_plain: %d tokens in one launch (max 65535)", n_tokens);
   dim3 grid(Hq, n_tokens);

@@ -51,6 +51,22 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// ---- cache layout -----------------------------------------------------------
+// A block of the cache holds block_size (a multiple of 16) slots of one KV head
+// as block_size/16 tiles of 16 slots x d elements, 16*d elements each, laid out
+// in the order the MFMA operands want them, so that a wave's load of a tile is
+// one contiguous run and LDS copies of it have no bank conflicts:
+//   K tile: [d/8][16 slots][8]      element (slot, e) at ((e/8)*16 + slot)*8 + e%8
+//   V tile: [d/16][4][16][4]        element (slot, e) at (((e/16)*4 + slot/4)*16 + e%16)*4 + slot%4
+// `off` is the slot inside the block; d is a multiple of 16.
+__host__ __device__ __forceinline__ size_t cache_k_index(int off, int e, int d) {
+  return (size_t)(off >> 4) * 16 * d + (size_t)(((e >> 3) * 16 + (off & 15)) * 8 + (e & 7));
+}
+__host__ __device__ __forceinline__ size_t cache_v_index(int off, int e, int d) {
+  const int s = off & 15;
+  return (size_t)(off >> 4) * 16 * d + (size_t)((((e >> 4) * 4 + (s >> 2)) * 16 + (e & 15)) * 4 + (s & 3));
+}
+
 // ---- host side -------------------------------------------------------------
 // One message slot per thread; ra_last_error() hands it to the caller.
 extern thread_local char ra_error_text[512];

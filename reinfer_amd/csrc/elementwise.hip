@@ -183,7 +183,8 @@ extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weigh
 //     rotation (crates/cuda/kernels/dense_kernels.cu:92-123; engine.rs:4122-4147)
 //   rotation: pairs (j, j + R/2) [style 0, half split] or (2j, 2j+1) [style 1],
 //     angle = pos * inv_freq[j] (dense_kernels.cu:125-139)
-//   cache: [block][kv head][slot in block][d]  (write: dense_kernels.cu:298-318)
+//   cache: [block][kv head][block_size * d] in the tiled order of cache_k_index /
+//     cache_v_index (write: dense_kernels.cu:298-318)
 // ---------------------------------------------------------------------------
 #define QK_WAVES 4
 #define QK_MAX_D 512
@@ -208,11 +209,12 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   const bool is_k = !is_q && head < Hq + Hkv;
   const int kvh = is_q ? 0 : (is_k ? head - Hq : head - Hq - Hkv);
   const int slot = slots[t];
-  TA* dst = nullptr;            // where a k or v head goes
+  TA* slab = nullptr;           // the (block, kv head) slab a k or v head goes to
+  int off = 0;                  // its slot there
   if (live && !is_q && slot >= 0) {
     const size_t blk = (size_t)(slot / block_size);
-    const int off = slot % block_size;
-    dst = (is_k ? kcache : vcache) + ((blk * Hkv + kvh) * block_size + off) * d;
+    off = slot % block_size;
+    slab = (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d;
   }
   float* b = buf[wave];
   float ss = 0.f;
@@ -226,8 +228,8 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   __syncthreads();
   if (!live) return;
   if (!is_q && !is_k) {          // v head: plain copy
-    if (dst)
-      for (int i = lane; i < d; i += RA_WAVE) dst[i] = from_f32<TA>(b[i]);
+    if (slab)
+      for (int i = lane; i < d; i += RA_WAVE) slab[cache_v_index(off, i, d)] = from_f32<TA>(b[i]);
     return;
   }
   const TW* w = is_q ? q_w : k_w;
@@ -236,8 +238,12 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
     ss = wave_sum(ss);
     rstd = rsqrtf(ss / (float)d + eps);
   }
-  TA* o = is_q ? u : dst;
-  if (!o) return;
+  if (!is_q && !slab) return;
+  // where element i of the head goes: in place for q, the cache slab for k
+  auto put = [&](int i, float v) {
+    if (is_q) u[i] = from_f32<TA>(v);
+    else slab[cache_k_index(off, i, d)] = from_f32<TA>(v);
+  };
   const float pos = (float)positions[t];
   const int half = rotary_dim / 2;
   for (int j = lane; j < half; j += RA_WAVE) {
@@ -250,13 +256,13 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
     }
     float sn, cs;
     sincosf(pos * inv_freq[j], &sn, &cs);
-    o[i0] = from_f32<TA>(a * cs - c * sn);
-    o[i1] = from_f32<TA>(a * sn + c * cs);
+    put(i0, a * cs - c * sn);
+    put(i1, a * sn + c * cs);
   }
   for (int i = rotary_dim + lane; i < d; i += RA_WAVE) {
     float a = b[i] * rstd;
     if (w) a *= to_f32(w[i]);
-    o[i] = from_f32<TA>(a);
+    put(i, a);
   }
 }
 
@@ -272,7 +278,9 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
            "qk_norm_rope_cache: rotary width %d must be even and <= head size %d", rotary_dim, d);
   RA_CHECK(rope_style == 0 || rope_style == 1, "qk_norm_rope_cache: unknown rotation style %d", rope_style);
   RA_CHECK((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_rope_cache: q and k norm weights go together");
-  RA_CHECK(block_size > 0, "qk_norm_rope_cache: block size %d", block_size);
+  RA_CHECK(block_size > 0 && block_size % 16 == 0 && d % 16 == 0,
+           "qk_norm_rope_cache: the cache is tiled 16 x 16: block size %d and head size %d must be multiples of 16",
+           block_size, d);
   RA_CHECK(n_tokens <= 65535, "qk_norm_rope_cache: %d tokens in one launch (max 65535)", n_tokens);
   dim3 grid((Hq + 2 * Hkv + QK_WAVES - 1) / QK_WAVES, n_tokens);
 #define RA_GO(TA, TW)                                                                              \

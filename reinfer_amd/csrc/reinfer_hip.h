@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 3
+#define RA_ABI_VERSION 5
 
 #ifdef __cplusplus
 extern "C" {
@@ -46,19 +46,24 @@ int ra_gemm_skinny_max_rows(void);
 int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                    int M, int N, int K, int lda, int ldc, hipStream_t stream);
 
-// bfloat16 flash-decode: one query per listed token, split-KV; partial buffers are
-// float [n_tokens, Hq, n_splits, d] and [n_tokens, Hq, n_splits, 2] (unused for one split)
-int ra_attention_decode_supports(int Hq, int Hkv, int d);
+// The cache of a layer: K and V are [blocks][Hkv][block_size * d], every (block, KV head) slab
+// in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);
+// block_size and d are multiples of 16.
+//
+// bfloat16 flash-decode: one query per listed token; keys in chunks of `chunk` (a multiple of
+// 128), max_chunks = chunks of the longest context. With more than one chunk: part_o float
+// [n_tokens * Hkv, max_chunks, G, d], part_ml float [.., 2], merged by a second kernel.
+int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size);
 int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                         const void* vcache, const int* block_tables, int max_blocks,
                         const int* token_list, const int* seq_of_token, const int* positions,
                         int n_tokens, int block_size, int Hq, int Hkv, int d, float scale, int window,
-                        int n_splits, float* part_o, float* part_ml, hipStream_t stream);
+                        int chunk, int max_chunks, float* part_o, float* part_ml, hipStream_t stream);
 
 // bfloat16 flash prefill over query tiles; tile_info holds 4 ints per tile:
 // request row in block_tables, first token row, number of queries (<= tile), first position
-int ra_attention_prefill_supports(int Hq, int Hkv, int d);
-int ra_attention_prefill_tile(void);
+int ra_attention_prefill_supports(int Hq, int Hkv, int d, int block_size);
+int ra_attention_prefill_tile(int Hq, int Hkv, int d);
 int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                          const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
                          int n_tiles, int block_size, int Hq, int Hkv, int d, float scale, int window,

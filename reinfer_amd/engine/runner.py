@@ -13,6 +13,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import torch
 
 from ..cache import CacheGroupSpec, CacheManager, OutOfBlocks, plan_groups
+from ..cache.layout import cache_shape
 from ..config import load_config
 from ..config.schema import ModelSpec
 from ..models import DecoderModel, declare_params
@@ -80,7 +81,8 @@ class ModelRunner:
         for i, (e, need) in enumerate(zip(spec.run_order, needs)):
             if isinstance(need, KVNeed):
                 if e.cache_from is None:
-                    shape = (self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
+                    # tiles of 16 slots in matrix-core operand order (cache/layout.py)
+                    shape = cache_shape(self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
                     k = torch.zeros(shape, dtype=dtype, device=device)
                     v = torch.zeros(shape, dtype=dtype, device=device)
                     self.caches.append(LayerCache(k=k, v=v, group=group_of[i], writes=True))

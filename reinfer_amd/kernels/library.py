@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 3
+ABI_VERSION = 5
 
 
 class KernelLibraryError(RuntimeError):
@@ -34,7 +34,7 @@ _SIGNATURES = {
     "ra_qk_norm_rope_cache": [P, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
     "ra_silu_mul": [P, P, I, I, I, I, P],
     "ra_attention_plain": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, P],
-    "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
+    "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P, P],
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
@@ -64,10 +64,11 @@ def load() -> ctypes.CDLL:
         lib.ra_sample_slices.argtypes = [c_int]
         for name in ("ra_attention_decode_supports", "ra_attention_prefill_supports"):
             getattr(lib, name).restype = c_int
-            getattr(lib, name).argtypes = [c_int, c_int, c_int]
-        for name in ("ra_attention_prefill_tile", "ra_gemm_skinny_max_rows"):
-            getattr(lib, name).restype = c_int
-            getattr(lib, name).argtypes = []
+            getattr(lib, name).argtypes = [c_int, c_int, c_int, c_int]
+        lib.ra_attention_prefill_tile.restype = c_int
+        lib.ra_attention_prefill_tile.argtypes = [c_int, c_int, c_int]
+        lib.ra_gemm_skinny_max_rows.restype = c_int
+        lib.ra_gemm_skinny_max_rows.argtypes = []
         if lib.ra_abi_version() != ABI_VERSION:
             raise KernelLibraryError(f"{path}: interface version {lib.ra_abi_version()}, expected {ABI_VERSION}; "
                                      "rebuild with `python -m reinfer_amd.csrc.build`")

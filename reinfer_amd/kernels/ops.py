@@ -97,10 +97,7 @@ class HipKernels:
         width = (num_heads + 2 * num_kv_heads) * head_dim
         if qkv.shape != (T, width) or not qkv.is_contiguous():
             raise ValueError(f"qk_norm_rope_cache: qkv {tuple(qkv.shape)}, expected [T, {width}] contiguous")
-        if kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[1] != num_kv_heads \
-                or kcache.shape[3] != head_dim or not kcache.is_contiguous() or not vcache.is_contiguous():
-            raise ValueError(f"qk_norm_rope_cache: cache {tuple(kcache.shape)} is not "
-                             f"[blocks, {num_kv_heads}, block, {head_dim}]")
+        self._check_cache("qk_norm_rope_cache", kcache, vcache, num_kv_heads, head_dim)
         if kcache.dtype != qkv.dtype or vcache.dtype != qkv.dtype:
             raise TypeError("qk_norm_rope_cache: the cache has the activations' dtype")
         _int32(positions, "positions", T)
@@ -118,7 +115,7 @@ class HipKernels:
         library.call("ra_qk_norm_rope_cache", qkv.data_ptr(), _tag(qkv, "qkv"), _ptr(q_weight),
                      _ptr(k_weight), wtag, float(eps), positions.data_ptr(), inv_freq.data_ptr(),
                      int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(),
-                     vcache.data_ptr(), kcache.shape[2], T, num_heads, num_kv_heads, head_dim, _stream())
+                     vcache.data_ptr(), kcache.shape[2] * 16, T, num_heads, num_kv_heads, head_dim, _stream())
 
     def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0) -> None:
         """out = silu(gate) * up. ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g
@@ -153,9 +150,11 @@ class HipKernels:
         if q.dtype != torch.bfloat16:
             return self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                         head_dim, scale, window, group)
-        plan = self._attention_plan(batch, q.device)
-        dec_ok = bool(lib.ra_attention_decode_supports(num_heads, num_kv_heads, head_dim))
-        pre_ok = bool(lib.ra_attention_prefill_supports(num_heads, num_kv_heads, head_dim))
+        bs = kcache.shape[2] * 16
+        tile = lib.ra_attention_prefill_tile(num_heads, num_kv_heads, head_dim)
+        plan = self._attention_plan(batch, q.device, tile)
+        dec_ok = bool(lib.ra_attention_decode_supports(num_heads, num_kv_heads, head_dim, bs))
+        pre_ok = bool(lib.ra_attention_prefill_supports(num_heads, num_kv_heads, head_dim, bs))
         if plan["n_decode"]:
             if dec_ok:
                 self.attention_decode(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
@@ -172,12 +171,15 @@ class HipKernels:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                      head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"])
 
-    def _attention_plan(self, batch, device):
-        """Which tokens go to which kernel; made once per step, shared by the layers."""
+    def _attention_plan(self, batch, device, tile: int):
+        """Which tokens go to which kernel; made once per step and query-tile size,
+        shared by the layers."""
         plan = batch.extra.get("attention_plan")
+        if plan is not None and plan.get("tile", tile) == tile:
+            return plan
+        plan = batch.extra.get(("attention_plan", tile))
         if plan is not None:
             return plan
-        tile = library.load().ra_attention_prefill_tile()
         dec, pre, tiles = [], [], []
         dec_max_ctx = 0
         t = 0
@@ -201,9 +203,20 @@ class HipKernels:
             "prefill_list": dev[n_dec_listed:n_dec_listed + len(pre)] if pre else None,
             "n_tiles": len(tiles) // 4,
             "tiles": dev[n_dec_listed + len(pre):] if tiles else None,
+            "tile": tile,
         }
-        batch.extra["attention_plan"] = plan
+        batch.extra[("attention_plan", tile)] = plan
         return plan
+
+    @staticmethod
+    def _check_cache(what: str, kcache, vcache, num_kv_heads: int, head_dim: int) -> None:
+        """K and V of a layer: [blocks, kv heads, block_size // 16, 16 * head_dim], tiled."""
+        if kcache.dim() != 4 or kcache.shape != vcache.shape or kcache.shape[1] != num_kv_heads \
+                or head_dim % 16 != 0 or kcache.shape[3] != 16 * head_dim \
+                or not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise ValueError(f"{what}: cache K {tuple(kcache.shape)}, V {tuple(vcache.shape)}: expected "
+                             f"[blocks, {num_kv_heads}, block_size // 16, 16 * {head_dim}] "
+                             "(head sizes in steps of 16)")
 
     def _check_attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim, group):
         _dev(q, out, kcache, vcache)
@@ -213,14 +226,14 @@ class HipKernels:
             raise ValueError(f"attention: out {tuple(out.shape)}, expected [{T}, {num_heads * head_dim}]")
         if q.shape[0] != T or q_stride < num_heads * head_dim or q.stride(0) != q_stride:
             raise ValueError("attention: query rows do not match the step's tokens")
-        if kcache.dtype != q.dtype or kcache.shape != vcache.shape or kcache.shape[1] != num_kv_heads \
-                or kcache.shape[3] != head_dim or not kcache.is_contiguous() or not vcache.is_contiguous():
-            raise ValueError("attention: cache does not match the layer's heads")
+        if kcache.dtype != q.dtype or vcache.dtype != q.dtype:
+            raise TypeError("attention: the cache has the activations' dtype")
+        self._check_cache("attention", kcache, vcache, num_kv_heads, head_dim)
         _int32(tables, "block tables")
         if tables.dim() != 2 or tables.shape[0] < batch.num_seqs:
             raise ValueError("attention: one block-table row per request of the step")
         # every key a query may read must have a table entry
-        if tables.shape[1] * kcache.shape[2] < batch.max_ctx_len:
+        if tables.shape[1] * kcache.shape[2] * 16 < batch.max_ctx_len:
             raise ValueError("attention: block tables shorter than the longest context")
         return tables
 
@@ -232,35 +245,42 @@ class HipKernels:
         library.call("ra_attention_plain", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), _tag(q, "attention"), tables.data_ptr(),
                      tables.shape[1], _ptr(token_list), batch.seq_of_token.data_ptr(),
-                     batch.positions.data_ptr(), n, kcache.shape[2], num_heads, num_kv_heads, head_dim,
+                     batch.positions.data_ptr(), n, kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,
                      float(scale), int(window), _stream())
 
     @staticmethod
-    def decode_splits(n_tokens: int, num_kv_heads: int, max_ctx: int) -> int:
-        """Split-KV factor: enough workgroups to fill 256 CUs a few times over, and
-        at least 256 keys a split."""
-        want = -(-1024 // max(1, n_tokens * num_kv_heads))
-        return max(1, min(want, max(1, max_ctx // 256), 64))
+    def decode_chunk(n_tokens: int, num_kv_heads: int, max_ctx: int):
+        """Keys per workgroup of the decode kernel, a multiple of 128: enough
+        workgroups to fill 256 CUs several times over. -> (chunk, chunks of max_ctx)"""
+        want = max(1, -(-2048 // max(1, n_tokens * num_kv_heads)))
+        chunk = -(-max_ctx // want)
+        chunk = max(128, -(-chunk // 128) * 128)
+        return chunk, max(1, -(-max_ctx // chunk))
 
     def attention_decode(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                          scale, window, group, token_list=None, n_listed=None, max_ctx=None,
-                         n_splits=None) -> None:
+                         chunk=None) -> None:
         tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, group)
         if q.dtype != torch.bfloat16:
             raise TypeError("attention_decode: bfloat16 only")
         n = batch.num_tokens if token_list is None else int(n_listed)
-        if n_splits is None:
-            n_splits = self.decode_splits(n, num_kv_heads, max_ctx or batch.max_ctx_len)
+        max_ctx = int(max_ctx or batch.max_ctx_len)
+        if chunk is None:
+            chunk, max_chunks = self.decode_chunk(n, num_kv_heads, max_ctx)
+        else:
+            max_chunks = max(1, -(-max_ctx // int(chunk)))
         part_o = part_ml = None
-        if n_splits > 1:
-            part_o = torch.empty((n, num_heads, n_splits, head_dim), dtype=torch.float32, device=q.device)
-            part_ml = torch.empty((n, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
+        if max_chunks > 1:
+            pairs = n * num_kv_heads
+            G = num_heads // num_kv_heads
+            part_o = torch.empty((pairs, max_chunks, G, head_dim), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((pairs, max_chunks, G, 2), dtype=torch.float32, device=q.device)
         library.call("ra_attention_decode", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
                      _ptr(token_list), batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), n,
-                     kcache.shape[2], num_heads, num_kv_heads, head_dim, float(scale), int(window),
-                     int(n_splits), _ptr(part_o), _ptr(part_ml), _stream())
+                     kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim, float(scale), int(window),
+                     int(chunk), int(max_chunks), _ptr(part_o), _ptr(part_ml), _stream())
 
     def attention_prefill(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                           scale, window, group, tiles, n_tiles) -> None:
@@ -271,7 +291,7 @@ class HipKernels:
         _int32(tiles, "query tiles", 4 * n_tiles)
         library.call("ra_attention_prefill", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
-                     tiles.data_ptr(), int(n_tiles), kcache.shape[2], num_heads, num_kv_heads, head_dim,
+                     tiles.data_ptr(), int(n_tiles), kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,
                      float(scale), int(window), _stream())
 
     # ---------------------------------------------------------------- linear

@@ -26,7 +26,8 @@ class StateNeed:
 class LayerCache:
     """The cache of one run-order entry, as its mixer sees it.
 
-    For keys and values: ``k``/``v`` are ``[blocks, kv_heads, block_size, head_dim]``,
+    For keys and values: ``k``/``v`` are ``[blocks, kv_heads, block_size // 16, 16 * head_dim]``,
+    tiles of 16 slots in the order of :mod:`reinfer_amd.cache.layout`;
     ``group`` picks the step's block tables and slots, ``writes`` is False for an
     entry that reads another entry's cache. For state: ``state`` is
     ``[max_seqs, *shape]``, indexed by the step's ``state_slots``.

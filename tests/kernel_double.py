@@ -11,6 +11,18 @@ from __future__ import annotations
 
 import torch
 
+from reinfer_amd.cache.layout import unpack_k, unpack_v
+
+
+def k_index(off, e, d):
+    """Element (slot off, e) of a (block, KV head) slab, as csrc/common.h cache_k_index."""
+    return (off >> 4) * 16 * d + ((e >> 3) * 16 + (off & 15)) * 8 + (e & 7)
+
+
+def v_index(off, e, d):
+    s = off & 15
+    return (off >> 4) * 16 * d + (((e >> 4) * 4 + (s >> 2)) * 16 + (e & 15)) * 4 + (s & 3)
+
 
 class KernelDouble:
     name = "cpu-double"
@@ -62,13 +74,15 @@ class KernelDouble:
         q = rot(norm(q, q_weight))
         k = rot(norm(k, k_weight))
         qkv.view(T, -1, d)[:, :num_heads] = q.to(qkv.dtype)
-        bs = kcache.shape[2]
+        bs = kcache.shape[2] * 16
+        kflat, vflat = kcache.view(kcache.shape[0], num_kv_heads, -1), vcache.view(vcache.shape[0], num_kv_heads, -1)
+        e = torch.arange(d)
         for t in range(T):
             s = int(slots[t])
             if s < 0:
                 continue
-            kcache[s // bs, :, s % bs, :] = k[t].to(kcache.dtype)
-            vcache[s // bs, :, s % bs, :] = v[t].to(vcache.dtype)
+            kflat[s // bs][:, k_index(s % bs, e, d)] = k[t].to(kcache.dtype)
+            vflat[s // bs][:, v_index(s % bs, e, d)] = v[t].to(vcache.dtype)
 
     GATE_GROUP = 8
 
@@ -89,7 +103,8 @@ class KernelDouble:
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                   scale, window, group):
         T = batch.num_tokens
-        bs = kcache.shape[2]
+        bs = kcache.shape[2] * 16
+        kl, vl = unpack_k(kcache, head_dim), unpack_v(vcache, head_dim)      # [blocks, Hkv, bs, d]
         tables = batch.block_tables[group]
         ratio = num_heads // num_kv_heads
         qh = q[:, :num_heads * head_dim].reshape(T, num_heads, head_dim).float()
@@ -99,8 +114,8 @@ class KernelDouble:
             lo = max(0, p - window + 1) if window > 0 else 0
             keys = torch.arange(lo, p + 1)
             blk = tables[seq, keys // bs].long()
-            K = kcache[blk, :, keys % bs, :].float()        # [n, Hkv, d]
-            V = vcache[blk, :, keys % bs, :].float()
+            K = kl[blk, :, keys % bs, :].float()        # [n, Hkv, d]
+            V = vl[blk, :, keys % bs, :].float()
             for a in range(num_heads):
                 s = (K[:, a // ratio, :] @ qh[t, a]) * scale
                 pr = torch.softmax(s, dim=0)

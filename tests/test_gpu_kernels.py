@@ -8,6 +8,7 @@ import torch
 
 import plain_qwen3 as plain
 from reinfer_amd import kernels
+from reinfer_amd.cache.layout import pack_k, pack_v, unpack_k, unpack_v
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -28,6 +29,16 @@ def close(got, ref, tol):
     err = (got - ref).abs().max().item()
     scale = ref.abs().max().item()
     assert err <= tol * max(scale, 1e-6), f"max error {err} against scale {scale}"
+
+
+def kt(kc):
+    """The tests build caches as [blocks, kv heads, slot, d]; the kernels take them in
+    tiles of 16 slots in matrix-core operand order."""
+    return pack_k(kc)
+
+
+def vt(vc):
+    return pack_v(vc)
 
 
 class FakeBatch:
@@ -142,7 +153,7 @@ def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm):
     positions = torch.tensor([0, 1, 15, 16, 17, 100, 255, 3, 4, 5, 6], dtype=torch.int32, device=DEV)
     slots_l = [5 * bs + 3, 0, 8 * bs + 15, -1, 2 * bs, 2 * bs + 1, 7 * bs + 9, 1 * bs + 1, 1 * bs + 2, 1 * bs + 3, 4 * bs]
     slots = torch.tensor(slots_l, dtype=torch.int32, device=DEV)
-    kc = torch.full((nblk, Hkv, bs, d), float("nan"), device=DEV, dtype=DT[dtype])
+    kc = torch.full((nblk, Hkv, bs // 16, 16 * d), float("nan"), device=DEV, dtype=DT[dtype])
     vc = torch.full_like(kc, float("nan"))
     j = torch.arange(max(rot // 2, 1), dtype=torch.float64)
     inv_freq = (theta ** (-2.0 * j / max(rot, 1))).float().to(DEV)
@@ -159,6 +170,7 @@ def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm):
         q_ref = rope_reference(q, positions.cpu(), theta, rot, style)
         k_ref = rope_reference(k, positions.cpu(), theta, rot, style)
     tol = OUT_TOL[dtype]
+    kc, vc = unpack_k(kc, d), unpack_v(vc, d)         # [blocks, kv heads, slot, d]
     close(qkv.view(T, -1, d)[:, :Hq], q_ref, tol)
     written = torch.zeros(nblk, bs, dtype=torch.bool)
     for t, s in enumerate(slots_l):
@@ -183,12 +195,12 @@ def test_rotation_depends_on_distance_only():
     dots = []
     for shift in (0, 37):
         qkv = base.clone()
-        kc = torch.zeros(4, Hkv, bs, d, device=DEV)
+        kc = torch.zeros(4, Hkv, bs // 16, 16 * d, device=DEV)
         vc = torch.zeros_like(kc)
         pos = torch.tensor([5 + shift, 9 + shift], dtype=torch.int32, device=DEV)
         slots = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
         ops().qk_norm_rope_cache(qkv, None, None, 0.0, pos, inv_freq, d, 0, slots, kc, vc, Hq, Hkv, d)
-        dots.append((qkv[1, :d] * kc[0, 0, 0]).sum().item())
+        dots.append((qkv[1, :d] * unpack_k(kc, d)[0, 0, 0]).sum().item())
     assert abs(dots[0] - dots[1]) < 1e-4 * max(1.0, abs(dots[0]))
 
 
@@ -254,7 +266,7 @@ def test_attention_plain(dtype, Hq, Hkv, d):
             T = sum(q_lens)
             out = torch.empty(T, Hq * d, device=DEV, dtype=DT[dtype])
             scale = 1.0 / math.sqrt(d)
-            ops().attention_plain(q.view(T, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hkv, d, scale, window, 0)
+            ops().attention_plain(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0)
             ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
             close(out, ref, OUT_TOL[dtype])
 
@@ -265,7 +277,7 @@ def test_attention_reduces_to_library_routine():
     q, kc, vc, tables = make_paged_case("float32", Hq, Hq, d, [n], [0], seed=5, poison=False)
     batch = FakeBatch([n], [0], tables)
     out = torch.empty(n, Hq * d, device=DEV)
-    ops().attention_plain(q.view(n, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hq, d, 1 / math.sqrt(d), 0, 0)
+    ops().attention_plain(q.view(n, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hq, d, 1 / math.sqrt(d), 0, 0)
     keys = torch.arange(n)
     K = kc[tables[0, keys // 16].long(), :, keys % 16, :].transpose(0, 1)     # [H, n, d]
     V = vc[tables[0, keys // 16].long(), :, keys % 16, :].transpose(0, 1)
@@ -430,7 +442,7 @@ def test_linear_dispatch_refuses_nothing_silently():
 DEC_SHAPES = [(4, 2, 16), (14, 2, 64), (12, 2, 48), (5, 5, 32), (8, 1, 128), (32, 8, 128), (2, 1, 256), (6, 3, 80)]
 DEC_BATCHES = [
     ([1], [0]), ([1], [15]), ([1], [16]), ([1, 1, 1], [31, 32, 700]), ([1] * 5, [63, 64, 65, 1000, 2]),
-    ([2, 1, 3, 1], [0, 257, 30, 99]),
+    ([2, 1, 3, 1], [0, 257, 30, 99]), ([1, 1, 1], [2047, 3000, 130]),
 ]
 
 
@@ -438,14 +450,14 @@ DEC_BATCHES = [
 def test_attention_decode(Hq, Hkv, d):
     for bi, (q_lens, starts) in enumerate(DEC_BATCHES):
         for window in (0, 19):
-            for n_splits in (1, 3, 8):
+            for chunk in (None, 128, 256, 1024):
                 q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=10 + bi)
                 batch = FakeBatch(q_lens, starts, tables)
                 T = sum(q_lens)
                 out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
                 scale = 1.0 / math.sqrt(d)
-                ops().attention_decode(q.view(T, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hkv, d, scale, window, 0,
-                                       n_splits=n_splits)
+                ops().attention_decode(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0,
+                                       chunk=chunk)
                 ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
                 close(out, ref, 2 ** -7)     # probabilities and values are bfloat16 products summed in float
 
@@ -458,7 +470,7 @@ def test_attention_decode_token_list_leaves_other_rows_alone():
     T = sum(q_lens)
     out = torch.full((T, Hq * d), 7.0, device=DEV, dtype=torch.bfloat16)
     lst = torch.tensor([0, 7], dtype=torch.int32, device=DEV)
-    ops().attention_decode(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0, lst, 2, 100)
+    ops().attention_decode(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0, lst, 2, 100)
     ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0)
     close(out[[0, 7]], ref[[0, 7]], 2 ** -7)
     assert (out[1:7] == 7.0).all()
@@ -473,7 +485,7 @@ PRE_BATCHES = [
 @pytest.mark.parametrize("Hq,Hkv,d", [(4, 2, 16), (14, 2, 64), (12, 2, 48), (5, 5, 32), (8, 1, 128), (32, 8, 128),
                                       (6, 3, 80), (3, 1, 112)])
 def test_attention_prefill(Hq, Hkv, d):
-    tile = 64
+    tile = kernels.library.load().ra_attention_prefill_tile(Hq, Hkv, d)
     for bi, (q_lens, starts) in enumerate(PRE_BATCHES):
         for window in (0, 19, 100):
             q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=20 + bi)
@@ -487,7 +499,7 @@ def test_attention_prefill(Hq, Hkv, d):
                 t += ql
             tiles = torch.tensor(info, dtype=torch.int32, device=DEV)
             scale = 1.0 / math.sqrt(d)
-            ops().attention_prefill(q.view(T, Hq * d), Hq * d, out, kc, vc, batch, Hq, Hkv, d, scale, window, 0,
+            ops().attention_prefill(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0,
                                     tiles, len(info) // 4)
             ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
             close(out, ref, 2 ** -7)
@@ -502,9 +514,10 @@ def test_attention_dispatch_mixed_batch():
     batch = FakeBatch(q_lens, starts, tables)
     T = sum(q_lens)
     out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
-    ops().attention(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0)
-    plan = batch.extra["attention_plan"]
-    assert plan["n_decode"] == 5 and plan["n_tiles"] == 3
+    ops().attention(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0)
+    tile = kernels.library.load().ra_attention_prefill_tile(Hq, Hkv, d)
+    plan = batch.extra[("attention_plan", tile)]
+    assert plan["n_decode"] == 5 and plan["n_tiles"] == -(-70 // tile) + 1
     close(out, attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0), 2 ** -7)
 
 
@@ -521,7 +534,7 @@ def test_far_key_among_hundreds_decode_and_prefill():
         batch = FakeBatch(q_lens, starts, tables)
         T = sum(q_lens)
         out = torch.empty((T, Hq * d), device=DEV, dtype=torch.bfloat16)
-        ops().attention(q.view(T, -1), Hq * d, out, kc, vc, batch, Hq, Hkv, d, d ** -0.5, 0, 0)
+        ops().attention(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0)
         ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0)
         assert ref[-1, :d].mean() > 4.0           # the far value dominates the reference
         close(out, ref, 2 ** -7)
