@@ -266,6 +266,71 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   }
 }
 
+// The same for the common shape (half-split rotation over the whole head, head
+// size a power of two between 16 and 256): one workgroup per token. The sines and
+// cosines of the token's angles are computed once, in LDS, for all heads (the
+// plain kernel computes them per head); a head is spread over d/8 lanes, each
+// holding rotation pairs (j..j+3, j+d/2..j+d/2+3) as two 4-element vectors.
+template <typename TA, typename TW, int LPH>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_cache_token_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w, const TW* __restrict__ k_w,
+                                float eps, const int* __restrict__ positions,
+                                const float* __restrict__ inv_freq, const int* __restrict__ slots,
+                                TA* __restrict__ kcache, TA* __restrict__ vcache, int block_size, int Hq,
+                                int Hkv, int d) {
+  __shared__ float cs[128], sn[128];
+  const int t = blockIdx.x;
+  const int half = d / 2;
+  const float pos = (float)positions[t];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) sincosf(pos * inv_freq[j], &sn[j], &cs[j]);
+  __syncthreads();
+  const int n_heads = Hq + 2 * Hkv;
+  const int sub = threadIdx.x / LPH, ln = threadIdx.x % LPH;
+  const int j0 = ln * 4;                       // pairs j0..j0+3
+  const int slot = slots[t];
+  const size_t blk = slot >= 0 ? (size_t)(slot / block_size) : 0;
+  const int off = slot >= 0 ? slot % block_size : 0;
+  for (int head = sub; head < n_heads; head += 256 / LPH) {
+    TA* u = qkv + ((size_t)t * n_heads + head) * d;
+    const bool is_q = head < Hq;
+    const bool is_k = !is_q && head < Hq + Hkv;
+    const int kvh = is_q ? 0 : (is_k ? head - Hq : head - Hq - Hkv);
+    if (!is_q && slot < 0) continue;           // nothing to store for this token
+    f32x4_raw a = Vec4<TA>::load(u + j0), c = Vec4<TA>::load(u + half + j0);
+    TA* slab = (is_q ? nullptr : (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d);
+    if (!is_q && !is_k) {                      // v head: copy into the V tile order
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        slab[cache_v_index(off, j0 + i, d)] = from_f32<TA>(a[i]);
+        slab[cache_v_index(off, half + j0 + i, d)] = from_f32<TA>(c[i]);
+      }
+      continue;
+    }
+    const TW* w = is_q ? q_w : k_w;
+    if (w) {
+      float ss = a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3] + c[0] * c[0] + c[1] * c[1] + c[2] * c[2] + c[3] * c[3];
+#pragma unroll
+      for (int m = LPH / 2; m > 0; m >>= 1) ss += __shfl_xor(ss, m, RA_WAVE);
+      const float rstd = rsqrtf(ss / (float)d + eps);
+      a = a * rstd * Vec4<TW>::load(w + j0);
+      c = c * rstd * Vec4<TW>::load(w + half + j0);
+    }
+    f32x4_raw ra, rc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ra[i] = a[i] * cs[j0 + i] - c[i] * sn[j0 + i];
+      rc[i] = a[i] * sn[j0 + i] + c[i] * cs[j0 + i];
+    }
+    if (is_q) {
+      Vec4<TA>::store(u + j0, ra);
+      Vec4<TA>::store(u + half + j0, rc);
+    } else {                                   // four elements of one 8-chunk are contiguous in the K tile
+      Vec4<TA>::store(slab + cache_k_index(off, j0, d), ra);
+      Vec4<TA>::store(slab + cache_k_index(off, half + j0, d), rc);
+    }
+  }
+}
+
 extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
                                      int weight_dtype, float eps, const int* positions,
                                      const float* inv_freq, int rotary_dim, int rope_style,
@@ -282,6 +347,32 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
            "qk_norm_rope_cache: the cache is tiled 16 x 16: block size %d and head size %d must be multiples of 16",
            block_size, d);
   RA_CHECK(n_tokens <= 65535, "qk_norm_rope_cache: %d tokens in one launch (max 65535)", n_tokens);
+  // the per-token kernel takes half-split rotation over the whole head, d in {16, 32, 64, 128, 256};
+  // with few tokens (decode) a wave per head spreads over more of the chip
+  const bool pow2 = (d & (d - 1)) == 0 && d >= 16 && d <= 256;
+  if (pow2 && n_tokens >= 32 && rope_style == 0 && rotary_dim == d && ((uintptr_t)qkv % 16) == 0 &&
+      (q_weight == nullptr || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0))) {
+#define RA_TOK2(TA, TW, LPH)                                                                              \
+  qk_norm_rope_cache_token_kernel<TA, TW, LPH><<<n_tokens, 256, 0, stream>>>(                             \
+      (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, slots, (TA*)kcache,  \
+      (TA*)vcache, block_size, Hq, Hkv, d)
+#define RA_TOK(TA, TW)                       \
+  do {                                       \
+    if (d == 16) RA_TOK2(TA, TW, 2);         \
+    else if (d == 32) RA_TOK2(TA, TW, 4);    \
+    else if (d == 64) RA_TOK2(TA, TW, 8);    \
+    else if (d == 128) RA_TOK2(TA, TW, 16);  \
+    else RA_TOK2(TA, TW, 32);                \
+  } while (0)
+    if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_TOK(float, float);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_TOK(bf16_t, bf16_t);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_TOK(bf16_t, float);
+    else return ra_fail("qk_norm_rope_cache: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
+#undef RA_TOK
+#undef RA_TOK2
+    RA_LAUNCH_CHECK("qk_norm_rope_cache");
+    return 0;
+  }
   dim3 grid((Hq + 2 * Hkv + QK_WAVES - 1) / QK_WAVES, n_tokens);
 #define RA_GO(TA, TW)                                                                              \
   qk_norm_rope_cache_kernel<TA, TW><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(                      \
@@ -317,12 +408,48 @@ __global__ void silu_mul_kernel(const TA* __restrict__ gu, TA* __restrict__ out,
   }
 }
 
+// eight outputs a thread, 16-byte loads and stores; I a multiple of 8, group 0 or a multiple of 8
+template <typename TA>
+__global__ void silu_mul_vec_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I, int group, size_t total8) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const int I8 = I / 8;
+  for (; idx < total8; idx += stride) {
+    const size_t t = idx / I8;
+    const int i = (int)(idx - t * I8) * 8;
+    const size_t gi = group > 0 ? (size_t)(i / group) * 2 * group + i % group : (size_t)i;
+    const size_t ui = group > 0 ? gi + group : (size_t)I + i;
+    const TA* row = gu + t * 2 * I;
+    f32x4_raw g0 = Vec4<TA>::load(row + gi), g1 = Vec4<TA>::load(row + gi + 4);
+    f32x4_raw u0 = Vec4<TA>::load(row + ui), u1 = Vec4<TA>::load(row + ui + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      g0[e] = g0[e] / (1.f + expf(-g0[e])) * u0[e];
+      g1[e] = g1[e] / (1.f + expf(-g1[e])) * u1[e];
+    }
+    Vec4<TA>::store(out + idx * 8, g0);
+    Vec4<TA>::store(out + idx * 8 + 4, g1);
+  }
+}
+
 extern "C" int ra_silu_mul(const void* gate_up, void* out, int act_dtype, int n_tokens, int intermediate,
                            int group, hipStream_t stream) {
   RA_CHECK(n_tokens > 0 && intermediate > 0, "silu_mul: empty input");
   RA_CHECK(group >= 0 && (group == 0 || intermediate % group == 0),
            "silu_mul: width %d is not a whole number of runs of %d", intermediate, group);
   const size_t total = (size_t)n_tokens * intermediate;
+  if (intermediate % 8 == 0 && group % 8 == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+      (act_dtype == RA_F32 || act_dtype == RA_BF16)) {
+    const size_t total8 = total / 8;
+    size_t vb = (total8 + 255) / 256;
+    if (vb > 65535 * 4) vb = 65535 * 4;
+    if (act_dtype == RA_F32)
+      silu_mul_vec_kernel<float><<<(unsigned)vb, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, group, total8);
+    else
+      silu_mul_vec_kernel<bf16_t><<<(unsigned)vb, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate, group, total8);
+    RA_LAUNCH_CHECK("silu_mul");
+    return 0;
+  }
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535 * 4) blocks = 65535 * 4;
   if (act_dtype == RA_F32)

@@ -120,6 +120,17 @@ def test_silu_mul(dtype):
     v = gu2.view(T, I2 // 3, 2, 3).double()
     g, u = v[:, :, 0].reshape(T, I2), v[:, :, 1].reshape(T, I2)
     close(out2, g / (1 + torch.exp(-g)) * u, OUT_TOL[dtype])
+    # widths in steps of 8 take the vector kernel: both layouts
+    I3 = 328
+    gu3 = gu[:, :2 * I3].contiguous()
+    out3 = torch.empty(T, I3, device=DEV, dtype=DT[dtype])
+    ops().silu_mul(gu3, out3)
+    g, u = gu3[:, :I3].double(), gu3[:, I3:].double()
+    close(out3, g / (1 + torch.exp(-g)) * u, OUT_TOL[dtype])
+    ops().silu_mul(gu3, out3, 8)
+    v = gu3.view(T, I3 // 8, 2, 8).double()
+    g, u = v[:, :, 0].reshape(T, I3), v[:, :, 1].reshape(T, I3)
+    close(out3, g / (1 + torch.exp(-g)) * u, OUT_TOL[dtype])
 
 
 def rope_reference(x, positions, theta, rotary_dim, style):
@@ -142,16 +153,23 @@ def rope_reference(x, positions, theta, rotary_dim, style):
 @pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [
     (4, 2, 16, 16, 0, True), (14, 2, 48, 48, 0, True), (5, 5, 128, 128, 0, True),
     (3, 1, 80, 32, 0, False), (6, 3, 64, 64, 1, True), (32, 8, 128, 128, 0, True), (2, 1, 256, 256, 0, True)])
-def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm):
+@pytest.mark.parametrize("T", [11, 45])       # few tokens: a wave per head; many: a workgroup per token
+def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm, T):
     torch.manual_seed(d + Hq)
-    T, bs, nblk, eps, theta = 11, 16, 9, 1e-6, 10000.0
+    bs, nblk, eps, theta = 16, 9, 1e-6, 10000.0
     width = (Hq + 2 * Hkv) * d
     qkv = torch.randn(T, width, device=DEV).to(DT[dtype])
     src = qkv.clone()
     qw = (torch.rand(d, device=DEV) + 0.5).to(DT[dtype]) if norm else None
     kw = (torch.rand(d, device=DEV) + 0.5).to(DT[dtype]) if norm else None
-    positions = torch.tensor([0, 1, 15, 16, 17, 100, 255, 3, 4, 5, 6], dtype=torch.int32, device=DEV)
+    pos_l = [0, 1, 15, 16, 17, 100, 255, 3, 4, 5, 6]
     slots_l = [5 * bs + 3, 0, 8 * bs + 15, -1, 2 * bs, 2 * bs + 1, 7 * bs + 9, 1 * bs + 1, 1 * bs + 2, 1 * bs + 3, 4 * bs]
+    g = torch.Generator().manual_seed(T)
+    free = [x for x in torch.randperm(nblk * bs, generator=g).tolist() if x not in slots_l]
+    while len(pos_l) < T:
+        pos_l.append(int(torch.randint(0, 128, (1,), generator=g)))   # float angles: their rounding grows with the position
+        slots_l.append(-1 if len(pos_l) % 7 == 0 else free.pop())
+    positions = torch.tensor(pos_l, dtype=torch.int32, device=DEV)
     slots = torch.tensor(slots_l, dtype=torch.int32, device=DEV)
     kc = torch.full((nblk, Hkv, bs // 16, 16 * d), float("nan"), device=DEV, dtype=DT[dtype])
     vc = torch.full_like(kc, float("nan"))
