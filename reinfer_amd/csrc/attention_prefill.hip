@@ -1,9 +1,11 @@
 // Paged flash attention for prompt portions, bfloat16, on the matrix cores.
 //
-// A workgroup (4 waves) takes one tile of consecutive query tokens of one
-// request and up to NC query heads that share a KV head. A wave owns NC column
-// tiles of 16: QT runs of 16 queries times HG heads (QT * HG <= NC), so every
-// key and value it reads from LDS feeds NC MFMAs. Keys and values come from the
+// A workgroup (8 waves, two a SIMD, so one wave's softmax arithmetic overlaps
+// the other's matrix products) takes one tile of consecutive query tokens of
+// one request and HG query heads that share a KV head: 8 * NC column tiles of
+// 16 columns, tile c = run c / HG of 16 queries, head c % HG; a wave owns NC
+// adjacent column tiles, so every key and value it reads from LDS feeds NC
+// MFMAs and all waves share one staged copy. Keys and values come from the
 // request's block table, earlier context and the portion's own tokens alike
 // (they were stored before this kernel runs), 64 keys a round, copied to LDS
 // as the cache holds them: tiles of 16 slots in MFMA operand order
@@ -25,8 +27,8 @@
 #include "common.h"
 #include "reinfer_hip.h"
 
-#define FP_THREADS 256
-#define FP_WAVES 4
+#define FP_THREADS 512
+#define FP_WAVES 8
 #define FP_KT 64          // keys per round
 
 __device__ __forceinline__ float fp_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -34,17 +36,15 @@ __device__ __forceinline__ float fp_exp2(float x) { return __builtin_amdgcn_exp2
 // how the heads of a group and the queries are spread over a wave's column tiles
 struct FpShape {
   int nc;      // column tiles a wave holds (template parameter)
-  int hg;      // heads of one KV head per workgroup
-  int qt;      // runs of 16 queries per wave
+  int hg;      // heads of one KV head per workgroup: 4, 2 or 1
+  int runs;    // runs of 16 queries per workgroup
 };
 static FpShape fp_shape(int Hq, int Hkv, int d) {
   FpShape s;
   const int G = Hq / Hkv;
-  s.nc = d <= 128 ? 4 : 2;
-  s.hg = 1;
-  for (int h = 1; h <= s.nc; ++h)
-    if (G % h == 0) s.hg = h;
-  s.qt = s.nc / s.hg;
+  s.nc = d <= 128 ? 2 : 1;
+  s.hg = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
+  s.runs = FP_WAVES * s.nc / s.hg;
   return s;
 }
 
@@ -54,7 +54,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
                      const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                      const int* __restrict__ block_tables, int max_blocks,
                      const int* __restrict__ tile_info,      // per tile: seq, first token row, n queries, first position
-                     int block_size, int Hq, int Hkv, int d, int HG, int QT, float scale_log2, int window) {
+                     int block_size, int Hq, int Hkv, int d, int HG, float scale_log2, int window) {
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   constexpr int NPRE = (FP_KT * DMAX / 8) / FP_THREADS;     // 16-byte chunks a thread fetches per operand
@@ -74,16 +74,16 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   const int pos0 = tile_info[tile * 4 + 3];
   const int* table = block_tables + (size_t)seq * max_blocks;
 
-  // column tile j of this wave: queries (wave * QT + j / HG) * 16 + r, head hgrp * HG + j % HG
-  const int n_real = QT * HG;
+  // column tile c = wave * NC + j: queries (c / HG) * 16 + r, head hgrp * HG + c % HG
   int qi[NC];
   bool q_live[NC];
   bf16x8_t qreg[NC][NDT];
 #pragma unroll
   for (int j = 0; j < NC; ++j) {
-    qi[j] = (wave * QT + j / HG) * 16 + r;
-    q_live[j] = j < n_real && qi[j] < nq;
-    const int head = kvh * G + hgrp * HG + j % HG;
+    const int c = wave * NC + j;
+    qi[j] = (c / HG) * 16 + r;
+    q_live[j] = qi[j] < nq;
+    const int head = kvh * G + hgrp * HG + c % HG;
     const bf16_t* qp = q + (size_t)(row0 + (q_live[j] ? qi[j] : 0)) * q_stride + (size_t)head * d;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
@@ -105,37 +105,40 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   const int last_pos = pos0 + nq - 1;
   const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const int kt_begin = first_key / FP_KT * FP_KT;
-  const int w_q0 = wave * QT * 16;                              // first query of the wave
+  const int w_q0 = (wave * NC / HG) * 16;                       // first query of the wave
+  const int w_qend = ((wave * NC + NC - 1) / HG + 1) * 16;      // one past its last
   const int w_first_pos = pos0 + w_q0;
-  const int w_last_pos = pos0 + min(w_q0 + QT * 16, nq) - 1;    // < w_first_pos if the wave has no query
+  const int w_last_pos = pos0 + min(w_qend, nq) - 1;            // < w_first_pos if the wave has no query
 
-  // fetch of one round into registers: the four 16-slot tiles of K and of V, chunk by chunk
-  const int tile_chunks = 2 * d;                 // 16-byte chunks of a tile
+  // fetch of one round into registers: the four 16-slot tiles of K and of V, 16 bytes a thread and
+  // step; tile tt_u of step u is the same for a whole wave, so its block id is a scalar load
+  constexpr int TCH = 2 * DMAX;                  // 16-byte chunks of a tile, padded to the template's head size
+  const int bs_shift = __builtin_ctz(block_size);      // block sizes are powers of two here
   bf16x8_t kpre[NPRE], vpre[NPRE];
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
       const int c = tid + u * FP_THREADS;
+      const int tt = __builtin_amdgcn_readfirstlane(c / TCH), w = c % TCH;
+      const int kt = k0 + tt * 16;
       const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
       kpre[u] = zero;
       vpre[u] = zero;
-      if (c < 4 * tile_chunks) {
-        const int tt = c / tile_chunks, w = c % tile_chunks;
-        const int kt = k0 + tt * 16;
-        if (kt <= last_pos && kt + 15 >= first_key) {
-          const int blk = table[kt / block_size];
-          const size_t src = ((size_t)blk * Hkv + kvh) * block_size * d + (size_t)((kt % block_size) >> 4) * 16 * d + w * 8;
-          kpre[u] = *(const bf16x8_t*)(kcache + src);
-          vpre[u] = *(const bf16x8_t*)(vcache + src);
-          // slots of the tile outside the visible range may hold anything (a freed block's bits): zero them
-          if (kt + 15 > last_pos || kt < first_key) {
-            const int kkey = kt + (w & 15);                      // K chunk w: 8 elements of slot w % 16
-            if (kkey > last_pos || kkey < first_key) kpre[u] = zero;
+      if (kt <= last_pos && kt + 15 >= first_key) {           // wave-uniform
+        const int blk = table[kt >> bs_shift];
+        const size_t tile_at = (((size_t)blk * Hkv + kvh) << bs_shift) * d + (size_t)((kt & (block_size - 1)) >> 4) * 16 * d;
+        if (w < 2 * d) {
+          kpre[u] = *(const bf16x8_t*)(kcache + tile_at + w * 8);
+          vpre[u] = *(const bf16x8_t*)(vcache + tile_at + w * 8);
+        }
+        // slots of the tile outside the visible range may hold anything (a freed block's bits): zero them
+        if (kt + 15 > last_pos || kt < first_key) {
+          const int kkey = kt + (w & 15);                      // K chunk w: 8 elements of slot w % 16
+          if (kkey > last_pos || kkey < first_key) kpre[u] = zero;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {                        // V chunk w: slots 4 ((w / 8) % 4) + e % 4
-              const int vkey = kt + ((w >> 3) & 3) * 4 + (e & 3);
-              if (vkey > last_pos || vkey < first_key) vpre[u][e] = (bf16_t)0.f;
-            }
+          for (int e = 0; e < 8; ++e) {                        // V chunk w: slots 4 ((w / 8) % 4) + e % 4
+            const int vkey = kt + ((w >> 3) & 3) * 4 + (e & 3);
+            if (vkey > last_pos || vkey < first_key) vpre[u][e] = (bf16_t)0.f;
           }
         }
       }
@@ -145,9 +148,10 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
       const int c = tid + u * FP_THREADS;
-      if (c < 4 * tile_chunks) {
-        *(bf16x8_t*)(Ks + c * 8) = kpre[u];
-        *(bf16x8_t*)(Vs + c * 8) = vpre[u];
+      const int tt = c / TCH, w = c % TCH;
+      if (w < 2 * d) {
+        *(bf16x8_t*)(Ks + (tt * 2 * d + w) * 8) = kpre[u];
+        *(bf16x8_t*)(Vs + (tt * 2 * d + w) * 8) = vpre[u];
       }
     }
   };
@@ -163,73 +167,81 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     if (w_last_pos < w_first_pos || w_last_pos < k0) continue;
     if (window > 0 && k0 + FP_KT - 1 < w_first_pos - window + 1) continue;
 
-    // scores S^T[key][column] for 4 sub-tiles of 16 keys
-    f32x4_t s[4][NC];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-      for (int j = 0; j < NC; ++j) s[ks][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        if (dt * 32 < d) {
-          const int e = dt * 32 + g * 8;
-          const bf16x8_t a = (e < d) ? *(const bf16x8_t*)(Ks + ks * 16 * d + ((dt * 4 + g) * 16 + r) * 8)
-                                     : (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-          for (int j = 0; j < NC; ++j)
-            s[ks][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j][dt], s[ks][j], 0, 0, 0);
-        }
-      }
-    }
-    // a round strictly inside every query's view needs no mask
-    const bool inner = k0 + FP_KT - 1 <= w_first_pos && w_q0 + QT * 16 <= nq && n_real == NC &&
-                       (window <= 0 || k0 >= w_last_pos - window + 1);
-    bf16x8_t pb[NC][2];
-#pragma unroll
-    for (int j = 0; j < NC; ++j) {
-      const int q_pos = pos0 + qi[j];
-      const int q_lo = (window > 0 && q_pos - window + 1 > 0) ? q_pos - window + 1 : 0;
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = s[ks][j][i] * scale_log2;
-          if (!inner) {
-            const int key = k0 + ks * 16 + 4 * g + i;
-            if (!(q_live[j] && key <= q_pos && key >= q_lo)) v = -INFINITY;
-          }
-          s[ks][j][i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
-      const float mn = fmaxf(m[j], tmax);
-      // a column with nothing visible so far keeps m = -inf and adds zeros
-      const float base = (mn == -INFINITY) ? 0.f : mn;
-      const float corr = (mn == -INFINITY) ? 1.f : fp_exp2(m[j] - mn);
-      float psum = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = fp_exp2(s[ks][j][i] - base);      // masked: exp2(-inf) = 0
-          psum += p;
-          pb[j][ks / 2][(ks % 2) * 4 + i] = from_f32<bf16_t>(p);
-        }
-      l[j] = l[j] * corr + psum;
-      m[j] = mn;
-      if (__any(corr != 1.f)) {
-#pragma unroll
-        for (int ot = 0; ot < NOT; ++ot)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[j][ot][i] *= corr;
-      }
-    }
-    // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
-    // k-slots (g, e): e < 4 -> key 4g + e of the first 16-key tile, e >= 4 -> of the second
+    // two halves of 32 keys, each: scores, online softmax, values
 #pragma unroll
     for (int kp = 0; kp < 2; ++kp) {
+      const int kh = k0 + kp * 32;
+      if (kh > w_last_pos) break;          // the second half may lie past the wave's last query
+      // scores S^T[key][column] for 2 sub-tiles of 16 keys
+      f32x4_t s[2][NC];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int j = 0; j < NC; ++j) s[ks][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          if (dt * 32 < d) {
+            const int e = dt * 32 + g * 8;
+            const bf16x8_t a = (e < d) ? *(const bf16x8_t*)(Ks + (kp * 2 + ks) * 16 * d + ((dt * 4 + g) * 16 + r) * 8)
+                                       : (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < NC; ++j)
+              s[ks][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j][dt], s[ks][j], 0, 0, 0);
+          }
+        }
+      }
+      // keys strictly inside every query's view need no mask
+      const bool inner = kh + 31 <= w_first_pos && w_qend <= nq &&
+                         (window <= 0 || kh >= w_last_pos - window + 1);
+      bf16x8_t pb[NC];
+#pragma unroll
+      for (int j = 0; j < NC; ++j) {
+        if (!inner) {
+          const int q_pos = pos0 + qi[j];
+          const int q_lo = (window > 0 && q_pos - window + 1 > 0) ? q_pos - window + 1 : 0;
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = kh + ks * 16 + 4 * g + i;
+              if (!(q_live[j] && key <= q_pos && key >= q_lo)) s[ks][j][i] = -INFINITY;
+            }
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(s[0][j][0], s[0][j][1]), fmaxf(s[0][j][2], s[0][j][3])),
+                           fmaxf(fmaxf(s[1][j][0], s[1][j][1]), fmaxf(s[1][j][2], s[1][j][3])));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
+        tmax *= scale_log2;                              // the scale is positive: it commutes with the maximum
+        // The running maximum follows the true one only when that has grown by more than 2^8:
+        // until then the probabilities are at most 256 times larger than with the true maximum,
+        // which float sums and bfloat16 operands hold as well, and the accumulators need no rescaling.
+        // The wave decides as a whole, so the rare rescaling is a uniform branch.
+        const bool grow = tmax > m[j] + 8.f;             // false for -inf maxima
+        if (__any(grow)) {
+          const float mn = fmaxf(m[j], tmax);
+          // a column with nothing visible so far keeps m = -inf and adds zeros
+          const float corr = (mn == -INFINITY) ? 1.f : fp_exp2(m[j] - mn);
+          l[j] *= corr;
+          m[j] = mn;
+#pragma unroll
+          for (int ot = 0; ot < NOT; ++ot)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][ot][i] *= corr;
+        }
+        const float base = (m[j] == -INFINITY) ? 0.f : m[j];
+        float psum = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = fp_exp2(fmaf(s[ks][j][i], scale_log2, -base));      // masked: exp2(-inf) = 0
+            psum += p;
+            pb[j][ks * 4 + i] = from_f32<bf16_t>(p);
+          }
+        l[j] += psum;
+      }
+      // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
+      // k-slots (g, e): e < 4 -> key 4g + e of the first 16-key tile, e >= 4 -> of the second
 #pragma unroll
       for (int ot = 0; ot < NOT; ++ot) {
         if (ot * 16 < d) {
@@ -239,7 +251,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
           const bf16x8_t a = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 #pragma unroll
           for (int j = 0; j < NC; ++j)
-            acc[j][ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[j][kp], acc[j][ot], 0, 0, 0);
+            acc[j][ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[j], acc[j][ot], 0, 0, 0);
         }
       }
     }
@@ -252,7 +264,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     lt += __shfl_xor(lt, 32, RA_WAVE);
     if (!q_live[j]) continue;
     const float inv = 1.f / lt;
-    const int head = kvh * G + hgrp * HG + j % HG;
+    const int head = kvh * G + hgrp * HG + (wave * NC + j) % HG;
     bf16_t* op = out + (size_t)(row0 + qi[j]) * out_stride + (size_t)head * d;
 #pragma unroll
     for (int ot = 0; ot < NOT; ++ot) {
@@ -268,13 +280,13 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 
 extern "C" int ra_attention_prefill_supports(int Hq, int Hkv, int d, int block_size) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return 0;
-  return (d % 16 == 0 && d >= 16 && d <= 256 && block_size > 0 && block_size % 16 == 0) ? 1 : 0;
+  return (d % 16 == 0 && d >= 16 && d <= 256 && block_size >= 16 && (block_size & (block_size - 1)) == 0) ? 1 : 0;
 }
 
 // queries per workgroup tile for these sizes
 extern "C" int ra_attention_prefill_tile(int Hq, int Hkv, int d) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || d <= 0) return 64;
-  return FP_WAVES * 16 * fp_shape(Hq, Hkv, d).qt;
+  return 16 * fp_shape(Hq, Hkv, d).runs;
 }
 
 extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride,
@@ -299,10 +311,10 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
   flash_prefill_kernel<DM, NCC><<<grid, FP_THREADS, 0, stream>>>(                                     \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, tile_info, block_size, Hq, Hkv, d, sh.hg,      \
-      sh.qt, scale_log2, window)
-  if (d <= 64) RA_FP(64, 4);
-  else if (d <= 128) RA_FP(128, 4);
-  else RA_FP(256, 2);
+      scale_log2, window)
+  if (d <= 64) RA_FP(64, 2);
+  else if (d <= 128) RA_FP(128, 2);
+  else RA_FP(256, 1);
 #undef RA_FP
   RA_LAUNCH_CHECK("attention_prefill");
   return 0;
