@@ -122,3 +122,163 @@ extern "C" int ra_sample(const float* logits, int n_rows, int vocab, int row_str
   RA_LAUNCH_CHECK("sample stage 2");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Filters and penalties, applied to a row of logits in place before ra_sample:
+//   frequency/presence: logit -= count * freq + pres for tokens among the last
+//     n of the request; repetition: logit > 0 divided, else multiplied by the
+//     penalty (crates/cuda/kernels/sampler_kernel.cu:207-221);
+//   then, on p = softmax(logit / T) and only if T > 0 (at T <= 0 the maximum
+//     survives every filter, sampler_kernel.cu:236-252):
+//   min_p: keep p >= min_p * max p; top_k: the k largest (value, then lower id);
+//   top_p: keep p >= theta, theta the largest value with
+//     sum_{kept, p >= theta} p >= top_p * (mass kept so far)
+//   (order and boundary rules: sampler_kernel.cu:20-43, 287-372). Removed
+//   tokens get -inf; ra_sample then applies the temperature and draws.
+// One workgroup per row; counts and sums are reduced in a fixed order.
+// ---------------------------------------------------------------------------
+#define FILTER_THREADS 1024
+
+__device__ __forceinline__ unsigned sortable(float v) {      // ascending order of floats as unsigned
+  const unsigned b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+template <typename T>
+__device__ __forceinline__ T filter_block_sum(T v, T* red) {
+#pragma unroll
+  for (int m = RA_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, RA_WAVE);
+  const int lane = threadIdx.x & (RA_WAVE - 1), wave = threadIdx.x / RA_WAVE;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  T t = 0;
+  for (int i = 0; i < FILTER_THREADS / RA_WAVE; ++i) t += red[i];
+  return t;
+}
+__device__ __forceinline__ float filter_block_max(float v, float* red) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & (RA_WAVE - 1), wave = threadIdx.x / RA_WAVE;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = -INFINITY;
+  for (int i = 0; i < FILTER_THREADS / RA_WAVE; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+struct FilterRow {           // one per row, in device memory
+  float temperature, top_p, min_p, repeat_penalty, frequency_penalty, presence_penalty;
+  int top_k, window_off, window_len, pad;
+};
+
+__global__ void __launch_bounds__(FILTER_THREADS)
+filter_logits_kernel(float* __restrict__ logits, int vocab, int row_stride, const FilterRow* __restrict__ rows,
+                     const int* __restrict__ window) {
+  __shared__ float redf[FILTER_THREADS / RA_WAVE];
+  __shared__ unsigned long long redu[FILTER_THREADS / RA_WAVE];
+  const FilterRow fr = rows[blockIdx.x];
+  float* lg = logits + (size_t)blockIdx.x * row_stride;
+  const int tid = threadIdx.x;
+
+  // penalties: the first occurrence of a token in the window carries its count
+  const bool pen = fr.repeat_penalty > 1.f || fr.frequency_penalty > 0.f || fr.presence_penalty > 0.f;
+  if (pen && fr.window_len > 0) {
+    const int* win = window + fr.window_off;
+    for (int w = tid; w < fr.window_len; w += FILTER_THREADS) {
+      const int tok = win[w];
+      if (tok < 0 || tok >= vocab) continue;
+      bool first = true;
+      int cnt = 0;
+      for (int x = 0; x < fr.window_len; ++x) {
+        if (win[x] == tok) {
+          if (x < w) { first = false; break; }
+          ++cnt;
+        }
+      }
+      if (!first) continue;
+      float l = lg[tok];
+      if (!isfinite(l)) continue;
+      l -= fr.frequency_penalty * (float)cnt + fr.presence_penalty;
+      if (fr.repeat_penalty > 1.f) l = l > 0.f ? l / fr.repeat_penalty : l * fr.repeat_penalty;
+      lg[tok] = l;
+    }
+    __syncthreads();
+  }
+  const float T = fr.temperature;
+  const bool use_k = fr.top_k > 0 && fr.top_k < vocab;
+  const bool use_p = fr.top_p > 0.f && fr.top_p < 1.f;
+  const bool use_m = fr.min_p > 0.f;
+  if (!(T > 0.f) || !(use_k || use_p || use_m)) return;
+
+  // x = logit / T; e = exp(x - max x) = p / max p
+  float mx = -INFINITY;
+  for (int v = tid; v < vocab; v += FILTER_THREADS) {
+    const float l = lg[v];
+    if (isfinite(l)) mx = fmaxf(mx, l / T);
+  }
+  mx = filter_block_max(mx, redf);
+  if (mx == -INFINITY) return;               // no finite logit: ra_sample reports it
+  // what is kept so far is described by two thresholds: e >= e_min and key >= key_min
+  float e_min = use_m ? fr.min_p : 0.f;      // min_p: p >= min_p * max p  <=>  e >= min_p
+  unsigned long long key_min = 0ull;
+  auto key_of = [&](int v, float x) { return ((unsigned long long)sortable(x) << 32) | (unsigned)(~v); };
+  if (use_k) {
+    // the k-th largest (value, lower id first) pair by bisection on the 64-bit key
+    unsigned long long lo = 0ull, hi = ~0ull;           // count(key >= lo) >= k > count(key >= hi)
+    for (int round = 0; round < 64 && hi - lo > 1ull; ++round) {
+      const unsigned long long mid = lo + (hi - lo) / 2ull;
+      unsigned long long c = 0ull;
+      for (int v = tid; v < vocab; v += FILTER_THREADS) {
+        const float l = lg[v];
+        if (isfinite(l) && key_of(v, l / T) >= mid) ++c;
+      }
+      c = filter_block_sum<unsigned long long>(c, redu);
+      if (c >= (unsigned long long)fr.top_k) lo = mid; else hi = mid;
+    }
+    key_min = lo;
+  }
+  float theta = 0.f;                          // top_p boundary on e
+  if (use_p) {
+    float zs = 0.f;
+    for (int v = tid; v < vocab; v += FILTER_THREADS) {
+      const float l = lg[v];
+      if (!isfinite(l)) continue;
+      const float x = l / T, e = __expf(x - mx);
+      if (e >= e_min && key_of(v, x) >= key_min) zs += e;
+    }
+    zs = filter_block_sum<float>(zs, redf);
+    const float need = fr.top_p * zs;
+    float flo = 0.f, fhi = 1.f;               // mass(e >= flo) >= need; e <= 1 always
+    for (int round = 0; round < 30; ++round) {
+      const float mid = 0.5f * (flo + fhi);
+      float mass = 0.f;
+      for (int v = tid; v < vocab; v += FILTER_THREADS) {
+        const float l = lg[v];
+        if (!isfinite(l)) continue;
+        const float x = l / T, e = __expf(x - mx);
+        if (e >= mid && e >= e_min && key_of(v, x) >= key_min) mass += e;
+      }
+      mass = filter_block_sum<float>(mass, redf);
+      if (mass >= need) flo = mid; else fhi = mid;
+    }
+    theta = flo;
+  }
+  for (int v = tid; v < vocab; v += FILTER_THREADS) {
+    const float l = lg[v];
+    if (!isfinite(l)) continue;
+    const float x = l / T, e = __expf(x - mx);
+    if (!(e >= e_min && e >= theta && key_of(v, x) >= key_min)) lg[v] = -INFINITY;
+  }
+}
+
+extern "C" int ra_filter_logits(float* logits, int n_rows, int vocab, int row_stride, const void* rows,
+                                const int* window, hipStream_t stream) {
+  RA_CHECK(n_rows > 0 && vocab > 0, "filter_logits: empty input (%d rows, vocabulary %d)", n_rows, vocab);
+  RA_CHECK(row_stride >= vocab, "filter_logits: row stride %d below the vocabulary %d", row_stride, vocab);
+  RA_CHECK(n_rows <= 65535, "filter_logits: %d rows in one launch (max 65535)", n_rows);
+  RA_CHECK(rows != nullptr, "filter_logits: no row parameters");
+  filter_logits_kernel<<<n_rows, FILTER_THREADS, 0, stream>>>(logits, vocab, row_stride, (const FilterRow*)rows, window);
+  RA_LAUNCH_CHECK("filter_logits");
+  return 0;
+}

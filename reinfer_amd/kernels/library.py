@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class KernelLibraryError(RuntimeError):
@@ -39,6 +39,7 @@ _SIGNATURES = {
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
+    "ra_filter_logits": [P, I, I, I, P, P, P],
 }
 
 

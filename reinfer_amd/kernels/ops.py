@@ -387,3 +387,31 @@ class HipKernels:
         library.call("ra_sample", logits.data_ptr(), n, V, logits.stride(0), temperature.data_ptr(),
                      seeds.data_ptr(), positions.data_ptr(), val.data_ptr(), idx.data_ptr(),
                      tokens.data_ptr(), _stream())
+
+    def filter_logits(self, logits: torch.Tensor, params, histories) -> None:
+        """Penalties and top-k / top-p / min-p of every row's SamplingParams, in place
+        (removed tokens become -inf); ``histories[i]`` are row i's tokens so far."""
+        import numpy as np
+        _dev(logits)
+        n, V = logits.shape
+        if logits.dtype != torch.float32 or logits.stride(1) != 1:
+            raise TypeError("filter_logits: logits are float32 rows")
+        rec = np.zeros((n, 10), dtype=np.float32)
+        irec = rec.view(np.int32)
+        window, off = [], 0
+        for i, (p, hist) in enumerate(zip(params, histories)):
+            rec[i, 0] = max(0.0, float(p.temperature))
+            rec[i, 1] = float(p.top_p or 0.0)
+            rec[i, 2] = float(p.min_p or 0.0)
+            rec[i, 3] = float(p.repeat_penalty or 0.0)
+            rec[i, 4] = max(0.0, float(p.frequency_penalty or 0.0))
+            rec[i, 5] = max(0.0, float(p.presence_penalty or 0.0))
+            irec[i, 6] = int(p.top_k or 0)
+            win = list(hist[-p.repeat_last_n:]) if (p.penalties and p.repeat_last_n > 0) else []
+            irec[i, 7], irec[i, 8] = off, len(win)
+            window += win
+            off += len(win)
+        rows_t = torch.from_numpy(rec).to(logits.device)
+        win_t = torch.tensor(window or [0], dtype=torch.int32).to(logits.device)
+        library.call("ra_filter_logits", logits.data_ptr(), n, V, logits.stride(0), rows_t.data_ptr(),
+                     win_t.data_ptr(), _stream())

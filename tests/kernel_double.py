@@ -131,6 +131,16 @@ class KernelDouble:
 
     linear_plain = linear
 
+    def filter_logits(self, logits, params, histories):
+        import plain_qwen3 as plain
+        for i, (p, hist) in enumerate(zip(params, histories)):
+            win = list(hist[-p.repeat_last_n:]) if p.repeat_last_n > 0 else []
+            logits[i] = plain.filter_logits(
+                logits[i], max(0.0, p.temperature), top_k=p.top_k or 0, top_p=p.top_p or 0.0,
+                min_p=p.min_p or 0.0, repeat_penalty=p.repeat_penalty or 0.0,
+                frequency_penalty=p.frequency_penalty or 0.0, presence_penalty=p.presence_penalty or 0.0,
+                window=win).float()
+
     def sample(self, logits, temperature, seeds, positions, tokens):
         from plain_qwen3 import mix64, splitmix64, unit_from_u64
         import math

@@ -203,3 +203,48 @@ def mix64(z: int) -> int:
 def unit_from_u64(x: int) -> float:
     """Top 24 bits over 2^24 (crates/cuda/kernels/sampler_kernel.cu:68-70)."""
     return (x >> 40) / 16777216.0
+
+
+def filter_logits(logits: torch.Tensor, temperature: float, *, top_k: int = 0, top_p: float = 0.0,
+                  min_p: float = 0.0, repeat_penalty: float = 0.0, frequency_penalty: float = 0.0,
+                  presence_penalty: float = 0.0, window: Sequence[int] = ()) -> torch.Tensor:
+    """Penalties, then the filters on softmax(logits / T); removed tokens are -inf.
+
+    Penalties (crates/cuda/kernels/sampler_kernel.cu:207-221): for a token that
+    occurs cnt > 0 times in the window, logit -= cnt * freq + pres, then logit > 0
+    is divided by the repetition penalty, else multiplied. Filters, if T > 0
+    (sampler_kernel.cu:20-43): min_p keeps p >= min_p * max p; top_k keeps the k
+    largest, lower id first among equals; top_p keeps, within what is left, the
+    values p >= theta with theta the largest value whose kept mass reaches
+    top_p times the mass left (ties at the boundary are all kept).
+    """
+    l = logits.clone().double()
+    V = l.numel()
+    if window and (repeat_penalty > 1 or frequency_penalty > 0 or presence_penalty > 0):
+        counts: Dict[int, int] = {}
+        for t in window:
+            counts[t] = counts.get(t, 0) + 1
+        for t, c in counts.items():
+            x = float(l[t])
+            x -= frequency_penalty * c + presence_penalty
+            if repeat_penalty > 1:
+                x = x / repeat_penalty if x > 0 else x * repeat_penalty
+            l[t] = x
+    if not temperature > 0:
+        return l
+    p = torch.softmax(l / temperature, dim=0)
+    keep = torch.ones(V, dtype=torch.bool)
+    if min_p > 0:
+        keep &= p >= min_p * p.max()
+    if 0 < top_k < V:
+        order = torch.sort(l, descending=True, stable=True).indices[:top_k]      # stable: lower id first among equals
+        kk = torch.zeros(V, dtype=torch.bool)
+        kk[order] = True
+        keep &= kk
+    if 0 < top_p < 1:
+        need = top_p * float(p[keep].sum())
+        vals, _ = torch.sort(p[keep], descending=True)
+        first = int((torch.cumsum(vals, dim=0) >= need).nonzero()[0])   # the largest theta whose mass reaches the need
+        keep &= p >= vals[first]
+    l[~keep] = float("-inf")
+    return l

@@ -402,6 +402,51 @@ def test_sample_distribution_is_softmax():
     assert ((freq - p).abs() <= 4 * torch.sqrt(p * (1 - p) / n) + 1e-4).all(), (freq, p)
 
 
+@pytest.mark.parametrize("V", [1000, 151936])
+def test_filter_logits_against_plain(V):
+    """Penalties, min-p, top-k and top-p against the plain chain; spaced logits keep every boundary clear."""
+    from reinfer_amd.sampling import SamplingParams
+    g = torch.Generator().manual_seed(V)
+    base = torch.randn(V, generator=g) * 3
+    cases = [
+        dict(temperature=0.7, top_k=5), dict(temperature=1.0, top_p=0.8), dict(temperature=1.3, min_p=0.05),
+        dict(temperature=0.9, top_k=40, top_p=0.5, min_p=0.01),
+        dict(temperature=1.0, repeat_penalty=1.3, frequency_penalty=0.4, presence_penalty=0.2, top_k=7),
+        dict(temperature=0.0, repeat_penalty=1.5, top_k=3),          # greedy: penalties only
+        dict(temperature=1.0, top_k=1),
+    ]
+    hist = torch.randint(0, V, (90,), generator=g).tolist()
+    hist += hist[:10] + [int(base.argmax())] * 3                    # repeats, and the favourite three times
+    params = [SamplingParams(**c) for c in cases]
+    logits = base.repeat(len(cases), 1).to(DEV)
+    logits[0, 17] = float("nan")                                     # a non-finite logit is never kept
+    ops().filter_logits(logits, params, [hist] * len(cases))
+    for i, c in enumerate(cases):
+        row = base.clone()
+        if i == 0:
+            row[17] = float("-inf")
+        kw = {k: v for k, v in c.items() if k != "temperature"}
+        ref = plain.filter_logits(row, c["temperature"], window=hist[-64:], **kw)
+        got = logits[i].cpu().double()
+        kept_ref, kept_got = torch.isfinite(ref), torch.isfinite(got)
+        if i == 0:
+            kept_got[17] = False
+        assert torch.equal(kept_ref, kept_got), (i, int(kept_ref.sum()), int(kept_got.sum()))
+        assert torch.allclose(got[kept_got], ref[kept_ref], rtol=1e-6, atol=1e-6)
+
+
+def test_filtered_sampling_stays_inside_top_k():
+    from reinfer_amd.sampling import Sampler, SamplingParams
+    V, n = 500, 300
+    torch.manual_seed(3)
+    row = torch.randn(V, device=DEV)
+    top = set(torch.topk(row, 4).indices.tolist())
+    sampler = Sampler(torch.device(DEV))
+    params = [SamplingParams(temperature=1.5, top_k=4)] * n
+    toks = sampler.sample(row.repeat(n, 1), params, list(range(n)), [7] * n, [[1, 2, 3]] * n)
+    assert set(toks) <= top and len(set(toks)) >= 3
+
+
 # ------------------------------------------------- bfloat16 kernels of serving
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 64])
 @pytest.mark.parametrize("N,K", [(100, 64), (333, 136), (1000, 96), (6144, 4096), (257, 520), (16, 8)])
