@@ -223,5 +223,8 @@ extern "C" int ra_gemm_skinny(const void* A, const void* W, const void* bias, vo
   RA_CHECK(out_dtype == RA_BF16 || out_dtype == RA_F32, "gemm_skinny: unknown output dtype tag %d", out_dtype);
   if (M <= 16) return launch_skinny<1, 1, 8, 4>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, stream);
   if (M <= 32) return launch_skinny<2, 1, 8, 4>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, stream);
+  // 33..64 rows: with few output features, 16 a workgroup keep all CUs busy; with many, 32 a
+  // workgroup halve the activations each one re-reads (measured at N = 4096 and 24576)
+  if (N <= 8192) return launch_skinny<4, 1, 8, 2>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, stream);
   return launch_skinny<4, 2, 8, 2>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, stream);
 }

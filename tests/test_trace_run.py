@@ -1,0 +1,55 @@
+"""bin/trace_run as a user runs it: a subprocess fed JSON steps on standard input, answering
+``done <step>`` after each and leaving ``<step>.f32`` files, compared with the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import TOL, make_folder, random_tokens, read_folder, rel_err
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_mixed_steps(tmp_path, dtype):
+    folder = make_folder(tmp_path, "B", "bfloat16")
+    raw, weights = read_folder(folder)
+    V = raw["vocab_size"]
+    seqs = {"a": random_tokens(70, V, 1), "b": random_tokens(41, V, 2), "c": random_tokens(50, V, 3)}
+    refs = {r: plain.forward(raw, weights, t) for r, t in seqs.items()}
+    # portions beside single tokens; c starts after a has ended, on a's blocks (192 tokens of cache)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": seqs["a"][:33], "want": [0, 32]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": seqs["a"][33:69], "want": list(range(36))},
+                                {"id": "b", "tokens": seqs["b"][:2], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": seqs["b"][2:40], "want": [37]},
+                                {"id": "a", "tokens": seqs["a"][69:70], "want": [0]}], "end": ["a"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": seqs["c"][:49], "want": []},
+                                {"id": "b", "tokens": seqs["b"][40:41], "want": [0]}], "end": ["b"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": seqs["c"][49:50], "want": [0]}], "end": ["c"]},
+    ]
+    out = tmp_path / f"out_{dtype}"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "192"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    fed = {r: 0 for r in seqs}
+    for s in steps:
+        want_rows = []
+        for e in s["entries"]:
+            want_rows += [refs[e["id"]][fed[e["id"]] + w] for w in e["want"]]
+            fed[e["id"]] += len(e["tokens"])
+        path = out / f"{s['step']}.f32"
+        if not want_rows:
+            assert not path.exists()
+            continue
+        got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(len(want_rows), V))
+        assert rel_err(got, torch.stack(want_rows)) < TOL[dtype]
