@@ -18,17 +18,20 @@
 // one is multiplied. The waves' partial sums are added through LDS in a fixed
 // order (deterministic; no atomics).
 //
-// Epilogues: plain (+ bias), or the SiLU gate of a feed-forward whose gate and
+// Epilogues: plain (+ bias); the SiLU gate of a feed-forward whose gate and
 // up rows are interleaved in groups of 8 (tile rows 0-7 gate, 8-15 up of the
 // same 8 features): out[m, 8*tile + j] = silu(gate_j) * up_j, which saves the
-// [M, 2I] round trip and a launch.
+// [M, 2I] round trip and a launch; or accumulation into a float matrix
+// (C += A . W^T: the residual add of an output projection).
+// (RMSNorm of a float input inside this kernel was tried and measured slower
+// than the separate norm kernel: every workgroup re-reads the rows in float.)
 //
 // The reference's own decode product is a thread-per-column split-K GEMV with a
 // second reduce launch (crates/cuda/kernels/gemm_m1.cu:63-235).
 #include "common.h"
 #include "reinfer_hip.h"
 
-enum { EPI_PLAIN = 0, EPI_SILU_PAIRS = 1 };
+enum { EPI_PLAIN = 0, EPI_SILU_PAIRS = 1, EPI_ACCUM = 2 };
 
 template <int MT, int NT, int WAVES, int U, int EPI, typename TO>
 __global__ void __launch_bounds__(WAVES * RA_WAVE)
@@ -160,7 +163,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mt * 16 + r;
-      if (EPI == EPI_PLAIN) {
+      if (EPI == EPI_ACCUM) {
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + nt * 16 + 4 * g + i;
+          if (n >= N) continue;
+          float v = acc[nt][mt][i];
+          if (bias) v += to_f32(bias[n]);
+          C[(size_t)m * ldc + n] = from_f32<TO>(to_f32(C[(size_t)m * ldc + n]) + v);   // this thread alone owns (m, n)
+        }
+      } else if (EPI == EPI_PLAIN) {
         if (m >= M) continue;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -198,6 +211,8 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
   if (epilogue == EPI_SILU_PAIRS) {
     if (out_dtype == RA_BF16) RA_GO(EPI_SILU_PAIRS, bf16_t);
     else RA_GO(EPI_SILU_PAIRS, float);
+  } else if (epilogue == EPI_ACCUM) {
+    RA_GO(EPI_ACCUM, float);
   } else {
     if (out_dtype == RA_BF16) RA_GO(EPI_PLAIN, bf16_t);
     else RA_GO(EPI_PLAIN, float);
@@ -214,7 +229,8 @@ extern "C" int ra_gemm_skinny(const void* A, const void* W, const void* bias, vo
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_skinny: empty product (%d, %d, %d)", M, N, K);
   RA_CHECK(M <= 64, "gemm_skinny: %d rows; this kernel takes at most 64", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_skinny: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
-  RA_CHECK(epilogue == EPI_PLAIN || epilogue == EPI_SILU_PAIRS, "gemm_skinny: unknown epilogue %d", epilogue);
+  RA_CHECK(epilogue == EPI_PLAIN || epilogue == EPI_SILU_PAIRS || epilogue == EPI_ACCUM, "gemm_skinny: unknown epilogue %d", epilogue);
+  RA_CHECK(epilogue != EPI_ACCUM || out_dtype == RA_F32, "gemm_skinny: accumulation is into a float matrix");
   const int n_out = epilogue == EPI_SILU_PAIRS ? N / 2 : N;
   RA_CHECK(epilogue != EPI_SILU_PAIRS || (N % 16 == 0 && bias == nullptr),
            "gemm_skinny: the gated epilogue needs N (%d) in whole tiles of 16 and no bias", N);

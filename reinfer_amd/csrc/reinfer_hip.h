@@ -41,7 +41,7 @@ int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int i
 
 // bfloat16, M <= 64, K and lda multiples of 8: weight-streaming MFMA product.
 // epilogue 0: C[M, N] = A . W^T (+ bias); epilogue 1: W rows are gate/up interleaved in runs of 8
-// and C[M, N/2] = silu(gate) * up
+// and C[M, N/2] = silu(gate) * up; epilogue 2: C is float and C += A . W^T (+ bias)
 int ra_gemm_skinny_max_rows(void);
 int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                    int M, int N, int K, int lda, int ldc, hipStream_t stream);

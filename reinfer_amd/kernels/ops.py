@@ -338,12 +338,22 @@ class HipKernels:
                      _tag(x, "linear input"), _tag(out, "linear output"), M, N, K, x.stride(0),
                      out.stride(0), _stream())
 
-    def linear_skinny(self, x, weight, out, bias=None) -> None:
+    def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False) -> None:
+        """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to."""
         M, N, K = self._check_linear(x, weight, out, bias)
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
+        if accumulate and out.dtype != torch.float32:
+            raise TypeError("linear_skinny: accumulation is into a float32 matrix")
         library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
-                     _tag(out, "linear output"), 0, M, N, K, x.stride(0), out.stride(0), _stream())
+                     _tag(out, "linear output"), 2 if accumulate else 0, M, N, K, x.stride(0), out.stride(0),
+                     _stream())
+
+    def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
+        """True if ``linear_skinny(..., accumulate=True)`` takes this product (out += x . W^T):
+        the residual add of an output projection then costs no kernel and no round trip."""
+        return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and x.shape[0] <= 64 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1)
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 

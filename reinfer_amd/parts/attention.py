@@ -24,6 +24,7 @@ from .registry import lookup, register_mixer
 @register_mixer("gqa_attention")
 class GroupedQueryAttention:
     graph_safe = True       # no host-side state: a decode step with it can be captured
+    adds_in_place = True    # forward(..., resid=) may add the output projection into the stream
 
     @classmethod
     def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
@@ -70,7 +71,7 @@ class GroupedQueryAttention:
     def cache_need(self) -> KVNeed:
         return KVNeed(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None):
         ops = kernels.current()
         T = x.shape[0]
         qkv = torch.empty((T, self.qkv_width), dtype=self.dtype, device=x.device)
@@ -82,6 +83,10 @@ class GroupedQueryAttention:
         attn = torch.empty((T, self.num_heads * self.head_dim), dtype=self.dtype, device=x.device)
         ops.attention(qkv, self.qkv_width, attn, cache.k, cache.v, batch, self.num_heads,
                       self.num_kv_heads, self.head_dim, self.scale, self.window, cache.group)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(attn, self.w_o):
+            ops.linear_skinny(attn, self.w_o, resid, accumulate=True)      # x += attn . Wo^T in the epilogue
+            return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(attn, self.w_o, out)
         return out

@@ -4,7 +4,8 @@
 (crates/cuda/src/engine.rs:4075-4314). The residual stream is float. A block
 gets the stream and the previous block's last addend, not yet added, so that
 the add and the norm are one kernel (the reference fuses the same pair for the
-o-projection, dense_kernels.cu:257-274); it returns its own last addend.
+o-projection, dense_kernels.cu:257-274); it returns its own last addend, or
+None if its last part added it into the stream itself.
 """
 from __future__ import annotations
 
@@ -42,7 +43,14 @@ class PreNormBlock:
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch,
                 cache: Optional[LayerCache]) -> torch.Tensor:
+        # A part that declares ``adds_in_place`` also gets the residual stream: where its last
+        # product can add into it, it does and returns None; any other part returns its addend.
         xn = self.mixer_norm.add_norm(resid, delta)
-        a = self.mixer.forward(xn, batch, cache)
+        if getattr(self.mixer, "adds_in_place", False):
+            a = self.mixer.forward(xn, batch, cache, resid=resid)
+        else:
+            a = self.mixer.forward(xn, batch, cache)
         xn = self.ffn_norm.add_norm(resid, a)
+        if getattr(self.ffn, "adds_in_place", False):
+            return self.ffn.forward(xn, batch, resid=resid)
         return self.ffn.forward(xn, batch)

@@ -9,7 +9,7 @@ A width that is no multiple of 8 keeps [gate; up] and the separate gate kernel.
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -22,6 +22,7 @@ from .registry import register_feed_forward
 @register_feed_forward("swiglu")
 class SwiGLU:
     graph_safe = True       # no host-side state: a decode step with it can be captured
+    adds_in_place = True    # forward(..., resid=) may add the down projection into the stream
 
     @classmethod
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
@@ -45,7 +46,7 @@ class SwiGLU:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + "down_proj.weight"]
 
-    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, batch, resid: Optional[torch.Tensor] = None):
         ops = kernels.current()
         T = x.shape[0]
         I = self.spec.intermediate
@@ -56,6 +57,10 @@ class SwiGLU:
             gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
             ops.linear(x, self.w_gate_up, gu)
             ops.silu_mul(gu, act)
+        can_add = getattr(ops, "can_accumulate", None)
+        if resid is not None and can_add and can_add(act, self.w_down):
+            ops.linear_skinny(act, self.w_down, resid, accumulate=True)    # x += act . Wd^T in the epilogue
+            return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(act, self.w_down, out)
         return out

@@ -100,6 +100,18 @@ class KernelDouble:
         self.linear(x, weight, gu)
         self.silu_mul(gu, out, self.GATE_GROUP)
 
+    # the accumulating epilogue, so that the parts' use of it runs on the CPU too
+    def can_accumulate(self, x, weight):
+        return x.shape[0] <= 64
+
+    def linear_skinny(self, x, weight, out, bias=None, accumulate=False):
+        if not accumulate:
+            return self.linear(x, weight, out, bias)
+        y = x.float() @ weight.float().T
+        if bias is not None:
+            y = y + bias.float()
+        out.add_(y.to(out.dtype))
+
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                   scale, window, group):
         T = batch.num_tokens

@@ -467,6 +467,11 @@ def test_linear_skinny(M, N, K, dout):
     ops().linear_skinny(x[M - 1:M], w, one)
     ops().linear_skinny(x, w, out)
     close(one, out[M - 1:M], 1e-6 if dout == "float32" else 2 ** -8)
+    # the accumulating epilogue: C += A . W^T into a float matrix
+    c0 = torch.randn(M, N, device=DEV)
+    c = c0.clone()
+    ops().linear_skinny(x, w, c, b, accumulate=True)
+    close(c, c0.double() + ref + b.double(), 1e-5)
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 20, 33, 64, 65, 200])

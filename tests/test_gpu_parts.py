@@ -108,7 +108,8 @@ def test_attention_part_with_rotation(dtype, Hq, Hkv, d, window):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_block_part(dtype):
+@pytest.mark.parametrize("n", [40, 7, 100])     # up to 64 rows the projections add into the stream in their epilogues
+def test_block_part(dtype, n):
     """Pre-norm arrangement: x += mixer(norm(x)); x += ffn(norm(x)), the last addend handed on."""
     h, Hq, Hkv, d, I, eps, theta = 80, 5, 1, 16, 104, 1e-5, 10000.0
     norm = NormSpec("rmsnorm", h, eps)
@@ -121,11 +122,10 @@ def test_block_part(dtype):
     block = cls(spec, w, DT[dtype], DEV)
     req = OneRequest(Hkv, d, dtype)
     torch.manual_seed(1)
-    n = 40
     x0 = torch.randn(n, h, device=DEV)
     resid = x0.clone()
-    delta = block.forward(resid, None, req.batch(n), req.cache)
-    got = resid.double().cpu() + delta.double().cpu()
+    delta = block.forward(resid, None, req.batch(n), req.cache)     # None: the last part added in place
+    got = resid.double().cpu() + (0 if delta is None else delta.double().cpu())
     x = x0.double().cpu()
     xn = plain.rms_norm(x, wd["L.input_layernorm.weight"], eps)
     x = x + plain.attention_block(xn, torch.arange(n), wd, "L.", Hq, Hkv, d, theta, eps, 0)
@@ -210,6 +210,7 @@ def test_toy_routed_feed_forward_and_position_in_a_block():
     resid_a, resid_b = x0[:20].clone(), x0[20:].clone()
     da = block.forward(resid_a, None, req.batch(20), req.cache)
     db = block.forward(resid_b, None, req.batch(13), req.cache)
+    assert da is not None and db is not None       # the toy feed-forward hands its addend back
     got = torch.cat([resid_a.double().cpu() + da.double().cpu(), resid_b.double().cpu() + db.double().cpu()])
 
     x = x0.double().cpu()
