@@ -19,7 +19,7 @@
 // Chunks of one (token, head) are merged by a second small kernel, always in
 // chunk order. (Merging in the last workgroup to arrive needs device-wide
 // release/acquire fences in every workgroup; on this chip each one writes back
-// and invalidates a whole L2, which made the kernel seven times slower.) A token
+// and invalidates a whole L2, which made the kernel nine times slower.) A token
 // whose keys fit one chunk is written directly.
 //
 // The reference's flash decode keeps the whole score row in shared memory,

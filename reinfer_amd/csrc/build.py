@@ -1,6 +1,7 @@
 """Builds the gfx950 kernel library with hipcc, in-tree, one object per source.
 
-``build()`` always compiles. ``ensure_built()`` compiles only when no library
+``build()`` always compiles (``build_host()`` likewise, the host runtime, with
+the host compiler). ``ensure_built()`` compiles only when no library
 is there or its sources changed since it was built; it prints a line per file
 meanwhile, since a first call in a fresh checkout takes a minute or so.
 """
@@ -150,5 +151,89 @@ def ensure_built() -> str:
     return build()
 
 
+# ---------------------------------------------------------------------------
+# The host runtime (cache bookkeeping, step packing, scheduler): plain C++ with
+# pybind11, built with the host compiler into the extension module reinfer_amd._host.
+# ---------------------------------------------------------------------------
+HOST_DIR = os.path.join(HERE, "host")
+HOST_SOURCES = ["host.cpp"]
+
+
+def _host_name() -> str:
+    import sysconfig
+    return "_host" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so")
+
+
+def host_hash() -> str:
+    h = hashlib.sha256()
+    for f in HOST_SOURCES:
+        with open(os.path.join(HOST_DIR, f), "rb") as fh:
+            h.update(fh.read())
+    h.update(sys.version.encode())
+    return h.hexdigest()
+
+
+def _host_dirs() -> List[str]:
+    pkg = os.path.dirname(HERE)
+    return [pkg, os.path.join(tempfile.gettempdir(), f"reinfer_amd_host_{os.getuid()}_{host_hash()[:12]}")]
+
+
+def build_host(verbose: bool = True) -> str:
+    import sysconfig
+    import pybind11
+    cxx = None
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/lib/llvm/bin/clang++"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            cxx = cand
+            break
+    if cxx is None:
+        raise RuntimeError("no C++ compiler found for the host runtime (set CXX)")
+    pkg, tmp = _host_dirs()
+    out_dir = pkg if os.access(pkg, os.W_OK) else tmp
+    os.makedirs(out_dir, exist_ok=True)
+    out = os.path.join(out_dir, _host_name())
+    part = out + f".{os.getpid()}.tmp"
+    cmd = [cxx, "-O2", "-shared", "-fPIC", "-std=c++17", "-fvisibility=hidden",
+           "-I", sysconfig.get_paths()["include"], "-I", pybind11.get_include(),
+           *[os.path.join(HOST_DIR, f) for f in HOST_SOURCES], "-o", part]
+    if verbose:
+        _say(f"compiling the host runtime with {cxx} (about 15 s) ...")
+    t0 = time.time()
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host runtime failed to compile:\n{r.stderr[-4000:]}")
+    os.replace(part, out)
+    with open(out + ".sha256", "w") as f:
+        f.write(host_hash())
+    if verbose:
+        _say(f"built {out} in {time.time() - t0:.0f} s")
+    return out
+
+
+def ensure_host_built() -> str:
+    want = host_hash()
+    stale = None
+    for d in _host_dirs():
+        path = os.path.join(d, _host_name())
+        if not os.path.isfile(path):
+            continue
+        try:
+            with open(path + ".sha256") as f:
+                if f.read().strip() == want:
+                    return path
+            stale = stale or path
+        except OSError:
+            return path          # a module without its stamp: take it as it is
+    try:
+        return build_host()
+    except Exception:
+        if stale is not None:
+            _say(f"warning: {stale} is older than its source and could not be rebuilt; using it")
+            return stale
+        raise
+
+
 if __name__ == "__main__":
     build()
+    build_host()

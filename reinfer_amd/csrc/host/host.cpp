@@ -1,0 +1,897 @@
+// The engine's host runtime: paged-cache bookkeeping, packing of a step's index
+// arrays, and the continuous-batching scheduler. Nothing here touches the GPU.
+// Python sees it as the extension module reinfer_amd._host (pybind11); the
+// classes in reinfer_amd/cache and reinfer_amd/engine/scheduler are these.
+//
+// Cache: keys and values live in blocks of block_size tokens. Layers with the
+// same needs form a group (all earlier keys, or a window of them); every group
+// has a pool of its own and every request one block table per group. Blocks are
+// taken lazily, when a step's tokens need them, given back when the request ends
+// or, in a window group, when the window has passed them, and used again, last
+// freed first (the reference's PagePool is LIFO the same way,
+// crates/memory/src/pool.rs:61-155). Beside the pools: slots for per-request
+// state of fixed size.
+//
+// Scheduler: each call of schedule() decides one step: every decoding request
+// takes one token first; what is left of the token budget goes to prompt
+// portions, requests already running before waiting ones, resumed ones before
+// new arrivals, then first come first served (crates/scheduler/src/batch.rs:69-101,
+// policy.rs:30-63). When blocks run out the newest running request that was not
+// preempted before is preempted and later recomputed from its prompt plus what
+// it generated (crates/scheduler/src/req.rs:340-357), so its output is what it
+// would have been. Everything is a pure function of the arrival order
+// (crates/scheduler/src/replay.rs:1-7).
+#include <pybind11/numpy.h>
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <deque>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace py = pybind11;
+
+// exception classes defined in Python (they carry attributes); set once at import, never destroyed
+static py::object* E_OutOfBlocks = nullptr;
+static py::object* E_OutOfSlots = nullptr;
+static py::object* E_RequestRefused = nullptr;
+
+[[noreturn]] static void raise_instance(const py::object& cls, const py::object& inst) {
+  PyErr_SetObject(cls.ptr(), inst.ptr());
+  throw py::error_already_set();
+}
+[[noreturn]] static void out_of_blocks(int group, int need, int free_) {
+  raise_instance(*E_OutOfBlocks, (*E_OutOfBlocks)(group, need, free_));
+}
+[[noreturn]] static void assertion(const std::string& msg) {
+  PyErr_SetString(PyExc_AssertionError, msg.c_str());
+  throw py::error_already_set();
+}
+static std::string show(const py::handle& o) { return py::repr(o).cast<std::string>(); }
+
+// ------------------------------------------------------------------- pools
+struct BlockPool {
+  int num_blocks;
+  std::vector<int> free_;          // back() is handed out next
+  std::vector<char> held;
+  long allocs = 0, frees = 0;
+
+  explicit BlockPool(int n) : num_blocks(n) {
+    if (n <= 0) throw py::value_error("a pool needs at least one block");
+    free_.reserve(n);
+    for (int b = n - 1; b >= 0; --b) free_.push_back(b);      // block 0 first
+    held.assign(n, 0);
+  }
+  int num_free() const { return (int)free_.size(); }
+  int num_held() const { return num_blocks - (int)free_.size(); }
+  int take() {
+    if (free_.empty()) out_of_blocks(-1, 1, 0);
+    const int b = free_.back();
+    free_.pop_back();
+    if (held[b]) assertion("block " + std::to_string(b) + " handed out twice");
+    held[b] = 1;
+    ++allocs;
+    return b;
+  }
+  void give_back(int b) {
+    if (b < 0 || b >= num_blocks) throw py::value_error("block " + std::to_string(b) + " is not of this pool");
+    if (!held[b]) throw std::runtime_error("block " + std::to_string(b) + " freed twice");
+    held[b] = 0;
+    free_.push_back(b);
+    ++frees;
+  }
+  void check() const {
+    std::vector<char> seen(num_blocks, 0);
+    int n_held = 0;
+    for (int b : free_) {
+      if (seen[b]) assertion("a block is on the free list twice");
+      seen[b] = 1;
+      if (held[b]) assertion("a free block is marked held");
+    }
+    for (char h : held) n_held += h;
+    if (n_held + (int)free_.size() != num_blocks) assertion("a block is lost");
+    if (allocs - frees != num_held()) assertion("allocations and frees do not add up");
+  }
+};
+
+struct SlotPool {
+  int num_slots;
+  std::vector<int> free_;
+  std::vector<char> held;
+  explicit SlotPool(int n) : num_slots(n) {
+    for (int s = n - 1; s >= 0; --s) free_.push_back(s);
+    held.assign(std::max(n, 0), 0);
+  }
+  int num_free() const { return (int)free_.size(); }
+  int take() {
+    if (free_.empty())
+      raise_instance(*E_OutOfSlots, (*E_OutOfSlots)("all " + std::to_string(num_slots) + " request slots are in use"));
+    const int s = free_.back();
+    free_.pop_back();
+    held[s] = 1;
+    return s;
+  }
+  void give_back(int s) {
+    if (s < 0 || s >= num_slots || !held[s]) throw std::runtime_error("slot " + std::to_string(s) + " freed twice");
+    held[s] = 0;
+    free_.push_back(s);
+  }
+};
+
+// ------------------------------------------------------------------ manager
+struct RequestCache {
+  int slot = 0;
+  int num_tokens = 0;                          // tokens whose keys are stored
+  std::vector<std::vector<int>> tables;        // per group; -1 = given back
+  std::vector<int> first_live;                 // per group: first block still held
+  bool fresh = true;                           // no step has run for it yet
+  uint64_t serial = 0;                         // distinguishes a request from an earlier one of the same id
+};
+
+struct KeyHash {
+  size_t operator()(const py::object& o) const { return (size_t)py::hash(o); }
+};
+struct KeyEq {
+  bool operator()(const py::object& a, const py::object& b) const { return a.equal(b); }
+};
+
+struct CacheManager {
+  py::list groups;                             // the CacheGroupSpec records, as given
+  std::vector<int> windows;
+  int block_size;
+  std::vector<BlockPool> pools;
+  SlotPool slots;
+  std::unordered_map<py::object, std::shared_ptr<RequestCache>, KeyHash, KeyEq> requests;
+  uint64_t next_serial = 1;
+
+  CacheManager(py::list groups_, int block_size_, std::vector<int> num_blocks, int max_seqs)
+      : groups(groups_), block_size(block_size_), slots(max_seqs) {
+    if (block_size <= 0) throw py::value_error("block_size must be positive");
+    if (num_blocks.size() != (size_t)py::len(groups)) throw py::value_error("one block count per cache group");
+    for (auto g : groups) windows.push_back(g.attr("window").cast<int>());
+    for (int n : num_blocks) pools.emplace_back(n);
+  }
+  int n_groups() const { return (int)windows.size(); }
+
+  std::shared_ptr<RequestCache> add(const py::object& rid) {
+    if (requests.count(rid)) throw py::key_error("request " + show(rid) + " is already live");
+    auto rc = std::make_shared<RequestCache>();
+    rc->slot = slots.take();
+    rc->tables.assign(n_groups(), {});
+    rc->first_live.assign(n_groups(), 0);
+    rc->serial = next_serial++;
+    requests.emplace(rid, rc);
+    return rc;
+  }
+  std::shared_ptr<RequestCache> get(const py::object& rid) const {
+    auto it = requests.find(rid);
+    if (it == requests.end()) throw py::key_error(show(rid));
+    return it->second;
+  }
+  bool contains(const py::object& rid) const { return requests.count(rid) != 0; }
+
+  // Give back everything a request holds, exactly once (crates/scheduler/src/req.rs:372-378).
+  void free(const py::object& rid) {
+    auto it = requests.find(rid);
+    if (it == requests.end()) throw py::key_error("request " + show(rid) + " is not live (freed twice?)");
+    auto rc = it->second;
+    requests.erase(it);
+    for (int g = 0; g < n_groups(); ++g) {
+      auto& t = rc->tables[g];
+      for (auto b = t.rbegin(); b != t.rend(); ++b)
+        if (*b >= 0) pools[g].give_back(*b);
+    }
+    slots.give_back(rc->slot);
+  }
+
+  // First block a query at first_query_pos can still read in group g.
+  int first_needed_block(int g, int first_query_pos) const {
+    const int w = windows[g];
+    if (w <= 0) return 0;
+    const int lo = first_query_pos - w + 1;
+    return std::max(0, lo) / block_size;
+  }
+  // Blocks each group must still take so that tokens [stored, new_total) fit.
+  void blocks_needed_into(const RequestCache& rc, int new_total, int* need) const {
+    const int want = (new_total + block_size - 1) / block_size;
+    for (int g = 0; g < n_groups(); ++g) {
+      const int have = (int)rc.tables[g].size();
+      // blocks wholly below the window of the first new query are never taken
+      const int first = std::max(have, first_needed_block(g, rc.num_tokens));
+      need[g] = std::max(0, want - first);
+    }
+  }
+  std::vector<int> blocks_needed(const py::object& rid, int new_total) const {
+    std::vector<int> need(n_groups());
+    blocks_needed_into(*get(rid), new_total, need.data());
+    return need;
+  }
+  bool can_grow(const std::vector<std::pair<py::object, int>>& growth) const {
+    std::vector<int> total(n_groups(), 0), need(n_groups());
+    for (auto& [rid, new_total] : growth) {
+      blocks_needed_into(*get(rid), new_total, need.data());
+      for (int g = 0; g < n_groups(); ++g) total[g] += need[g];
+    }
+    for (int g = 0; g < n_groups(); ++g)
+      if (total[g] > pools[g].num_free()) return false;
+    return true;
+  }
+  // Take the blocks for tokens up to new_total; all groups or none.
+  void grow_rc(RequestCache& rc, int new_total) {
+    if (new_total < rc.num_tokens) throw py::value_error("a request's cache does not shrink");
+    std::vector<int> need(n_groups());
+    blocks_needed_into(rc, new_total, need.data());
+    for (int g = 0; g < n_groups(); ++g)
+      if (need[g] > pools[g].num_free()) out_of_blocks(g, need[g], pools[g].num_free());
+    const int want = (new_total + block_size - 1) / block_size;
+    for (int g = 0; g < n_groups(); ++g) {
+      auto& table = rc.tables[g];
+      const int first = first_needed_block(g, rc.num_tokens);
+      while ((int)table.size() < want) {
+        if ((int)table.size() < first) {
+          table.push_back(-1);                 // below the window from the start: never held
+          rc.first_live[g] = (int)table.size();
+        } else {
+          table.push_back(pools[g].take());
+        }
+      }
+    }
+  }
+  void grow(const py::object& rid, int new_total) { grow_rc(*get(rid), new_total); }
+
+  // The step has stored tokens up to new_total; give back what every later query's window has passed.
+  void commit_rc(RequestCache& rc, int new_total) {
+    rc.num_tokens = new_total;
+    rc.fresh = false;
+    for (int g = 0; g < n_groups(); ++g) {
+      const int first = first_needed_block(g, new_total);       // the next query sits at new_total
+      auto& table = rc.tables[g];
+      const int end = std::min(first, (int)table.size());
+      for (int b = rc.first_live[g]; b < end; ++b)
+        if (table[b] >= 0) {
+          pools[g].give_back(table[b]);
+          table[b] = -1;
+        }
+      rc.first_live[g] = std::max(rc.first_live[g], end);
+    }
+  }
+  void commit(const py::object& rid, int new_total) { commit_rc(*get(rid), new_total); }
+
+  // Flat cache slot (block * block_size + offset) of position pos; -1 if not held.
+  int slot_of(const py::object& rid, int group, int pos) const {
+    auto rc = get(rid);
+    const int b = rc->tables.at(group).at(pos / block_size);
+    return b < 0 ? -1 : b * block_size + pos % block_size;
+  }
+
+  // No block lost, held twice or free while held.
+  void check() const {
+    for (int g = 0; g < n_groups(); ++g) {
+      pools[g].check();
+      std::vector<char> seen(pools[g].num_blocks, 0);
+      int n = 0;
+      for (auto& kv : requests)
+        for (int b : kv.second->tables[g])
+          if (b >= 0) {
+            if (seen[b]) assertion("group " + std::to_string(g) + ": a block is held by two requests");
+            if (!pools[g].held[b]) assertion("group " + std::to_string(g) + ": a table names a free block");
+            seen[b] = 1;
+            ++n;
+          }
+      if (n != pools[g].num_held())
+        assertion("group " + std::to_string(g) + ": " + std::to_string(pools[g].num_held()) + " held, " +
+                  std::to_string(n) + " in tables");
+    }
+    std::vector<char> seen(std::max(slots.num_slots, 0), 0);
+    for (auto& kv : requests) {
+      if (seen[kv.second->slot]) assertion("a state slot is held twice");
+      seen[kv.second->slot] = 1;
+    }
+    if ((int)requests.size() + slots.num_free() != slots.num_slots) assertion("a state slot is lost");
+  }
+
+  py::dict stats() const {
+    py::dict d;
+    py::list total, free_, allocs, frees;
+    for (auto& p : pools) {
+      total.append(p.num_blocks);
+      free_.append(p.num_free());
+      allocs.append(p.allocs);
+      frees.append(p.frees);
+    }
+    d["block_size"] = block_size;
+    d["live_requests"] = (int)requests.size();
+    d["blocks_total"] = total;
+    d["blocks_free"] = free_;
+    d["allocs"] = allocs;
+    d["frees"] = frees;
+    return d;
+  }
+
+  // ------------------------------------------------------ a step's index arrays
+  // Sizes of the packed int32 buffer of a step over `entries` (objects with rid, tokens, want):
+  // -> (q_lens, starts, widths per group, wanted rows). The layout itself is the caller's.
+  py::tuple step_shape(const py::list& entries) const {
+    std::vector<int> q_lens, starts, widths(n_groups(), 1);
+    int n_out = 0;
+    for (auto e : entries) {
+      auto rc = get(e.attr("rid").cast<py::object>());
+      q_lens.push_back((int)py::len(e.attr("tokens")));
+      starts.push_back(rc->num_tokens);
+      n_out += (int)py::len(e.attr("want"));
+      for (int g = 0; g < n_groups(); ++g) widths[g] = std::max(widths[g], (int)rc->tables[g].size());
+    }
+    return py::make_tuple(q_lens, starts, widths, n_out);
+  }
+
+  // Fill the packed buffer. `offs` holds the first element of: tokens, positions, request of each
+  // token, first token of each request (n + 1), start, context length, state slot, fresh flag,
+  // wanted rows, "store nothing" slots, then per group the block tables [n, width] and after all
+  // tables per group the cache slot of each token.
+  void fill_step(const py::list& entries, py::array_t<int32_t, py::array::c_style> buffer,
+                 const std::vector<long>& offs, const std::vector<int>& widths) const {
+    auto h = buffer.mutable_unchecked<1>();
+    const int n = (int)py::len(entries), G = n_groups();
+    if ((int)offs.size() != 10 + 2 * G || (int)widths.size() != G) throw py::value_error("fill_step: bad layout");
+    const long o_tok = offs[0], o_pos = offs[1], o_seq = offs[2], o_cu = offs[3], o_start = offs[4], o_ctx = offs[5],
+               o_state = offs[6], o_fresh = offs[7], o_rows = offs[8], o_noslot = offs[9];
+    long t = 0, r = 0;
+    int i = 0;
+    for (auto e : entries) {
+      auto rc = get(e.attr("rid").cast<py::object>());
+      const int start = rc->num_tokens;
+      int q = 0;
+      for (auto tok : e.attr("tokens")) {
+        h(o_tok + t + q) = tok.cast<int32_t>();
+        h(o_pos + t + q) = start + q;
+        h(o_seq + t + q) = i;
+        h(o_noslot + t + q) = -1;
+        ++q;
+      }
+      h(o_cu + i) = (int32_t)t;
+      h(o_start + i) = start;
+      h(o_ctx + i) = start + q;
+      h(o_state + i) = rc->slot;
+      h(o_fresh + i) = rc->fresh ? 1 : 0;
+      for (auto w : e.attr("want")) h(o_rows + r++) = (int32_t)(t + w.cast<int>());
+      for (int g = 0; g < G; ++g) {
+        const auto& table = rc->tables[g];
+        const long row = offs[10 + g] + (long)i * widths[g];
+        // entries given back (-1) are never read by a kernel; 0 keeps every index valid
+        for (size_t b = 0; b < table.size(); ++b) h(row + (long)b) = table[b] >= 0 ? table[b] : 0;
+        const long o_slot = offs[10 + G + g];
+        for (int j = 0; j < q; ++j) {
+          const int pos = start + j;
+          const int blk = table.at(pos / block_size);
+          h(o_slot + t + j) = blk < 0 ? -1 : blk * block_size + pos % block_size;
+        }
+      }
+      t += q;
+      ++i;
+    }
+    h(o_cu + n) = (int32_t)t;
+  }
+};
+
+// Rows of a captured decode step: which request sits in which row of the static buffers, and how
+// much of its block tables is already there, so that a step writes only what changed.
+struct DecodeRows {
+  std::shared_ptr<CacheManager> manager;
+  int B, W;
+  std::vector<long> offs;       // token_ids, positions, start_pos, ctx_lens, state_slots, fresh, sample_pos,
+                                // temps, seeds (in int32 units), then per group: table, slots
+  std::vector<uint64_t> owner;  // serial of the request in each row, 0 = padding
+  std::vector<std::vector<int>> row_len;
+
+  DecodeRows(std::shared_ptr<CacheManager> m, int B_, int W_, std::vector<long> offs_)
+      : manager(std::move(m)), B(B_), W(W_), offs(std::move(offs_)) {
+    if ((int)offs.size() != 9 + 2 * manager->n_groups()) throw py::value_error("DecodeRows: bad layout");
+    owner.assign(B, 0);
+    row_len.assign(manager->n_groups(), std::vector<int>(B, 0));
+  }
+
+  void pad(int32_t* h, int lo, int hi) {
+    const int G = manager->n_groups();
+    for (int i = lo; i < hi; ++i) {
+      h[offs[0] + i] = 0;       // token 0 at position 0 that stores nothing
+      h[offs[1] + i] = 0;
+      h[offs[2] + i] = 0;
+      h[offs[3] + i] = 1;
+      h[offs[4] + i] = -1;
+      h[offs[5] + i] = 0;
+      h[offs[6] + i] = 0;
+      h[offs[7] + i] = 0;       // temperature 0.0f
+      h[offs[8] + 2 * i] = 0;
+      h[offs[8] + 2 * i + 1] = 0;
+      for (int g = 0; g < G; ++g) h[offs[9 + 2 * g + 1] + i] = -1;
+      owner[i] = 0;
+    }
+  }
+
+  // entries: objects with rid and tokens (one each); sampling: None or (temperatures, seeds, positions)
+  void fill(const py::list& entries, py::array_t<int32_t, py::array::c_style> buffer, const py::object& sampling) {
+    int32_t* h = buffer.mutable_data();
+    const int n = (int)py::len(entries), G = manager->n_groups(), bs = manager->block_size;
+    if (n > B) throw py::value_error("DecodeRows: more entries than rows");
+    int i = 0;
+    for (auto e : entries) {
+      auto rc = manager->get(e.attr("rid").cast<py::object>());
+      const int p = rc->num_tokens;
+      h[offs[0] + i] = (*e.attr("tokens").begin()).cast<int32_t>();
+      h[offs[1] + i] = p;
+      h[offs[2] + i] = p;
+      h[offs[3] + i] = p + 1;
+      h[offs[4] + i] = rc->slot;
+      h[offs[5] + i] = rc->fresh ? 1 : 0;
+      const bool same = owner[i] == rc->serial;
+      for (int g = 0; g < G; ++g) {
+        const auto& table = rc->tables[g];
+        if ((int)table.size() > W) throw py::value_error("DecodeRows: block table longer than the static row");
+        const int have = same ? row_len[g][i] : 0;
+        int32_t* row = h + offs[9 + 2 * g] + (long)i * W;
+        // entries given back (-1) are never read; 0 keeps every index valid
+        for (int b = have; b < (int)table.size(); ++b) row[b] = table[b] >= 0 ? table[b] : 0;
+        row_len[g][i] = (int)table.size();
+        const int blk = table.at(p / bs);
+        h[offs[9 + 2 * g + 1] + i] = blk < 0 ? -1 : blk * bs + p % bs;
+      }
+      owner[i] = rc->serial;
+      ++i;
+    }
+    if (!sampling.is_none()) {
+      auto s = sampling.cast<py::tuple>();
+      int k = 0;
+      for (auto v : s[0]) {
+        const float f = v.cast<float>();
+        std::memcpy(h + offs[7] + k++, &f, 4);
+      }
+      k = 0;
+      for (auto v : s[1]) {
+        const int64_t x = v.cast<int64_t>();
+        std::memcpy(h + offs[8] + 2 * k++, &x, 8);
+      }
+      k = 0;
+      for (auto v : s[2]) h[offs[6] + k++] = v.cast<int32_t>();
+    } else {
+      for (int k = 0; k < n; ++k) {
+        h[offs[6] + k] = 0;
+        h[offs[7] + k] = 0;
+        h[offs[8] + 2 * k] = 0;
+        h[offs[8] + 2 * k + 1] = 0;
+      }
+    }
+    int hi = n;
+    for (int k = B - 1; k >= n; --k)
+      if (owner[k] != 0) {
+        hi = k + 1;
+        break;
+      }
+    if (hi > n) pad(h, n, hi);
+  }
+  void pad_all(py::array_t<int32_t, py::array::c_style> buffer) { pad(buffer.mutable_data(), 0, B); }
+};
+
+// --------------------------------------------------------------- scheduler
+static const char* WAITING = "waiting";
+static const char* RUNNING = "running";
+static const char* FINISHED = "finished";
+
+struct Request {
+  py::object rid;
+  std::vector<int> prompt;
+  py::object params;
+  py::object seed;
+  long arrival = 0;
+  std::string state = WAITING;
+  std::vector<int> output;
+  int num_computed = 0;            // tokens of prompt + output whose keys are in the cache
+  bool resumed = false;            // preempted at least once
+  py::object finish_reason = py::none();
+  int preemptions = 0;
+  // read once from params
+  int max_tokens = 0;
+  bool ignore_eos = false;
+  std::vector<int> stop_ids;
+
+  int num_tokens() const { return (int)(prompt.size() + output.size()); }
+  int remaining() const { return num_tokens() - num_computed; }
+  // in the cache up to its last token, which is a generated one
+  bool decoding() const { return state == RUNNING && !output.empty() && remaining() == 1; }
+  std::vector<int> tokens() const {
+    std::vector<int> t(prompt);
+    t.insert(t.end(), output.begin(), output.end());
+    return t;
+  }
+  int token_at(int i) const {
+    if (i < 0 || i >= num_tokens()) throw py::index_error("token index out of range");
+    return i < (int)prompt.size() ? prompt[i] : output[i - prompt.size()];
+  }
+  std::vector<int> tokens_slice(int start, int n) const {
+    std::vector<int> t;
+    t.reserve(std::max(n, 0));
+    for (int i = start; i < start + n; ++i) t.push_back(token_at(i));
+    return t;
+  }
+};
+using RequestP = std::shared_ptr<Request>;
+
+struct Portion {
+  RequestP request;
+  int start, length;
+  // the portion reaches the request's current end: its last logits give a token
+  bool samples() const { return start + length == request->num_tokens(); }
+};
+
+struct StepPlan {
+  std::vector<Portion> portions;
+  std::vector<RequestP> preempted;
+  std::vector<RequestP> finished;      // ended without running (cache)
+  int num_tokens() const {
+    int n = 0;
+    for (auto& p : portions) n += p.length;
+    return n;
+  }
+};
+
+struct Scheduler {
+  std::shared_ptr<CacheManager> manager;
+  int max_num_seqs, budget, max_model_len, max_chunk;
+  std::vector<int> eos;
+  std::deque<RequestP> waiting;
+  std::vector<RequestP> running;
+  std::unordered_map<py::object, RequestP, KeyHash, KeyEq> requests;
+  long arrivals = 0;
+  long c_steps = 0, c_preemptions = 0, c_finished = 0, c_refused = 0, c_tokens = 0;
+
+  Scheduler(std::shared_ptr<CacheManager> m, int max_num_seqs_, int max_num_batched_tokens, int max_model_len_,
+            py::object max_chunk_, std::vector<int> eos_ids)
+      : manager(std::move(m)), budget(max_num_batched_tokens), max_model_len(max_model_len_), eos(std::move(eos_ids)) {
+    if (max_num_seqs_ < 1 || max_num_batched_tokens < 1)
+      throw py::value_error("max_num_seqs and max_num_batched_tokens must be positive");
+    max_num_seqs = std::min(max_num_seqs_, manager->slots.num_slots);
+    max_chunk = (max_chunk_.is_none() || max_chunk_.cast<int>() <= 0) ? max_num_batched_tokens : max_chunk_.cast<int>();
+  }
+
+  [[noreturn]] void refuse(const std::string& why, bool count = true) {
+    if (count) ++c_refused;
+    raise_instance(*E_RequestRefused, (*E_RequestRefused)(why));
+  }
+  int pool_tokens() const {
+    int n = manager->pools.at(0).num_blocks;
+    for (auto& p : manager->pools) n = std::min(n, p.num_blocks);
+    return n * manager->block_size;
+  }
+
+  RequestP add(const py::object& rid, const std::vector<int>& prompt, const py::object& params, const py::object& seed) {
+    auto it = requests.find(rid);
+    if (it != requests.end() && it->second->state != FINISHED) refuse("request " + show(rid) + " is already live", false);
+    const int n = (int)prompt.size();
+    if (n == 0) refuse("empty prompt");
+    if (n + 1 > max_model_len)
+      refuse("prompt of " + std::to_string(n) + " tokens leaves no room in a context of " + std::to_string(max_model_len));
+    if (n + 1 > pool_tokens())
+      refuse("prompt of " + std::to_string(n) + " tokens can never fit a cache of " + std::to_string(pool_tokens()) + " tokens");
+    auto req = std::make_shared<Request>();
+    req->rid = rid;
+    req->prompt = prompt;
+    req->params = params;
+    req->seed = seed;
+    req->arrival = arrivals++;
+    req->max_tokens = params.attr("max_tokens").cast<int>();
+    req->ignore_eos = params.attr("ignore_eos").cast<bool>();
+    for (auto t : params.attr("stop_token_ids")) req->stop_ids.push_back(t.cast<int>());
+    requests[rid] = req;
+    waiting.push_back(req);
+    return req;
+  }
+
+  // Idempotent; frees once (crates/scheduler/src/req.rs:326-338).
+  bool abort(const py::object& rid) {
+    auto it = requests.find(rid);
+    if (it == requests.end() || it->second->state == FINISHED) return false;
+    auto req = it->second;
+    if (req->state == RUNNING) {
+      running.erase(std::find(running.begin(), running.end(), req));
+      manager->free(rid);
+    } else {
+      waiting.erase(std::find(waiting.begin(), waiting.end(), req));
+    }
+    req->state = FINISHED;
+    req->finish_reason = py::str("abort");
+    return true;
+  }
+  bool has_work() const { return !waiting.empty() || !running.empty(); }
+
+  void preempt(const RequestP& req, StepPlan& plan) {
+    running.erase(std::find(running.begin(), running.end(), req));
+    manager->free(req->rid);
+    req->state = WAITING;
+    req->num_computed = 0;
+    req->resumed = true;
+    ++req->preemptions;
+    ++c_preemptions;
+    waiting.push_front(req);
+    plan.preempted.push_back(req);
+  }
+
+  StepPlan schedule() {
+    StepPlan plan;
+    const int G = manager->n_groups();
+    int left = budget;
+    std::vector<int> need(G), one(G), free_(G);
+    auto read_free = [&]() {
+      for (int g = 0; g < G; ++g) free_[g] = manager->pools[g].num_free();
+    };
+
+    // 1. decoding requests: one token each; make room by preempting the newest
+    while (true) {
+      std::fill(need.begin(), need.end(), 0);
+      int n_dec = 0;
+      for (auto& r : running)
+        if (r->decoding()) {
+          ++n_dec;
+          manager->blocks_needed_into(*manager->get(r->rid), r->num_computed + 1, one.data());
+          for (int g = 0; g < G; ++g) need[g] += one[g];
+        }
+      read_free();
+      bool is_short = n_dec > left;
+      for (int g = 0; g < G; ++g) is_short = is_short || need[g] > free_[g];
+      if (!is_short) break;
+      if (running.size() == 1) {
+        auto lone = running[0];
+        running.clear();
+        manager->free(lone->rid);
+        lone->state = FINISHED;
+        lone->finish_reason = py::str("cache");
+        ++c_finished;
+        plan.finished.push_back(lone);
+        break;
+      }
+      // victims: not yet preempted first, newest arrival first (policy.rs:59-63)
+      RequestP victim = running[0];
+      for (auto& r : running)
+        if (std::make_pair(r->resumed, -r->arrival) < std::make_pair(victim->resumed, -victim->arrival)) victim = r;
+      preempt(victim, plan);
+    }
+    std::vector<RequestP> by_arrival(running);
+    std::sort(by_arrival.begin(), by_arrival.end(), [](const RequestP& a, const RequestP& b) { return a->arrival < b->arrival; });
+    read_free();
+    for (auto& r : by_arrival)
+      if (r->decoding()) {
+        manager->blocks_needed_into(*manager->get(r->rid), r->num_computed + 1, one.data());
+        for (int g = 0; g < G; ++g) free_[g] -= one[g];
+        plan.portions.push_back(Portion{r, r->num_computed, 1});
+        --left;
+      }
+
+    // Largest portion <= want whose blocks are free (leaving `reserve` blocks in every group); takes them from free_.
+    const int bs = manager->block_size;
+    auto fit = [&](const RequestP& req, int start, int want, bool live, int reserve) {
+      int n = want;
+      while (n > 0) {
+        if (live) {
+          manager->blocks_needed_into(*manager->get(req->rid), start + n, one.data());
+        } else {
+          for (int g = 0; g < G; ++g) one[g] = (start + n + bs - 1) / bs;
+        }
+        bool ok = true;
+        for (int g = 0; g < G; ++g) ok = ok && one[g] + reserve <= free_[g];
+        if (ok) {
+          for (int g = 0; g < G; ++g) free_[g] -= one[g];
+          return n;
+        }
+        // shrink to the last block edge that fits
+        n = std::min(n - 1, ((start + n - 1) / bs) * bs - start);
+      }
+      return 0;
+    };
+
+    // 2. prompt portions of running requests, oldest first
+    for (auto& r : by_arrival) {
+      if (r->decoding()) continue;
+      if (left <= 0) break;
+      const int n = fit(r, r->num_computed, std::min({r->remaining(), max_chunk, left}), true, 0);
+      if (n > 0) {
+        plan.portions.push_back(Portion{r, r->num_computed, n});
+        left -= n;
+      }
+    }
+
+    // 3. admissions: resumed first (they sit at the head), then arrival order
+    while (!waiting.empty() && left > 0 && (int)running.size() < max_num_seqs) {
+      auto r = waiting.front();
+      if (std::find(plan.preempted.begin(), plan.preempted.end(), r) != plan.preempted.end())
+        break;                      // preempted in this very step: not before the next
+      // a block of headroom for every running request, so that an admission does not force a
+      // preemption at the very next step
+      const int n = fit(r, 0, std::min({r->remaining(), max_chunk, left}), false, (int)running.size());
+      if (n == 0) break;            // first come first served: nobody overtakes
+      waiting.pop_front();
+      manager->add(r->rid);
+      r->state = RUNNING;
+      running.push_back(r);
+      plan.portions.push_back(Portion{r, 0, n});
+      left -= n;
+    }
+
+    // requests keep their order in the batch: by arrival (batch.rs:13-15 sorts by id)
+    std::stable_sort(plan.portions.begin(), plan.portions.end(),
+                     [](const Portion& a, const Portion& b) { return a.request->arrival < b.request->arrival; });
+    ++c_steps;
+    c_tokens += plan.num_tokens();
+    return plan;
+  }
+
+  // The step ran: advance cursors, append sampled tokens, finish and free. Order of the checks:
+  // stop ids, then the cap on new tokens, then the context (crates/scheduler/src/req.rs:281-314);
+  // the stop token is consumed, not emitted.
+  std::vector<RequestP> complete(const StepPlan& plan, const py::dict& sampled) {
+    std::vector<RequestP> done;
+    for (auto& p : plan.portions) {
+      auto& r = p.request;
+      const bool samples = p.samples();        // before the cursor and the output move
+      r->num_computed = p.start + p.length;
+      if (!samples) continue;
+      const int tok = sampled[r->rid].cast<int>();
+      const bool is_eos = std::find(eos.begin(), eos.end(), tok) != eos.end();
+      const bool stop = (is_eos && !r->ignore_eos) ||
+                        std::find(r->stop_ids.begin(), r->stop_ids.end(), tok) != r->stop_ids.end();
+      if (stop) {
+        r->finish_reason = py::str("stop");
+      } else {
+        r->output.push_back(tok);
+        if ((int)r->output.size() >= r->max_tokens) r->finish_reason = py::str("length");
+        else if (r->num_tokens() >= max_model_len) r->finish_reason = py::str("length");
+      }
+      if (!r->finish_reason.is_none()) {
+        r->state = FINISHED;
+        running.erase(std::find(running.begin(), running.end(), r));
+        manager->free(r->rid);
+        ++c_finished;
+        done.push_back(r);
+      }
+    }
+    return done;
+  }
+
+  py::dict counters() const {
+    py::dict d;
+    d["steps"] = c_steps;
+    d["preemptions"] = c_preemptions;
+    d["finished"] = c_finished;
+    d["refused"] = c_refused;
+    d["tokens"] = c_tokens;
+    return d;
+  }
+};
+
+PYBIND11_MODULE(_host, m) {
+  m.doc() = "host runtime of reinfer_amd: cache bookkeeping, step packing, scheduler";
+  m.def("set_exceptions", [](py::object oob, py::object oos, py::object refused) {
+    E_OutOfBlocks = new py::object(std::move(oob));
+    E_OutOfSlots = new py::object(std::move(oos));
+    E_RequestRefused = new py::object(std::move(refused));
+  });
+  m.attr("WAITING") = WAITING;
+  m.attr("RUNNING") = RUNNING;
+  m.attr("FINISHED") = FINISHED;
+
+  py::class_<BlockPool>(m, "BlockPool", "Fixed set of block ids with a LIFO free list; every misuse is an error.")
+      .def(py::init<int>(), py::arg("num_blocks"))
+      .def_readonly("num_blocks", &BlockPool::num_blocks)
+      .def_property_readonly("num_free", &BlockPool::num_free)
+      .def_property_readonly("num_held", &BlockPool::num_held)
+      .def_readonly("allocs", &BlockPool::allocs)
+      .def_readonly("frees", &BlockPool::frees)
+      .def("take", &BlockPool::take)
+      .def("give_back", &BlockPool::give_back)
+      .def("is_held", [](const BlockPool& p, int b) { return b >= 0 && b < p.num_blocks && p.held[b]; })
+      .def("check", &BlockPool::check);
+
+  py::class_<SlotPool>(m, "SlotPool", "Ids for per-request state of fixed size.")
+      .def(py::init<int>(), py::arg("num_slots"))
+      .def_readonly("num_slots", &SlotPool::num_slots)
+      .def_property_readonly("num_free", &SlotPool::num_free)
+      .def("take", &SlotPool::take)
+      .def("give_back", &SlotPool::give_back);
+
+  py::class_<RequestCache, std::shared_ptr<RequestCache>>(m, "RequestCache")
+      .def_readonly("slot", &RequestCache::slot)
+      .def_readwrite("num_tokens", &RequestCache::num_tokens)
+      .def_readonly("tables", &RequestCache::tables)
+      .def_readonly("first_live", &RequestCache::first_live)
+      .def_readwrite("fresh", &RequestCache::fresh);
+
+  py::class_<CacheManager, std::shared_ptr<CacheManager>>(m, "CacheManager")
+      .def(py::init<py::list, int, std::vector<int>, int>(), py::arg("groups"), py::arg("block_size"),
+           py::arg("num_blocks"), py::arg("max_seqs"))
+      .def_readonly("groups", &CacheManager::groups)
+      .def_readonly("block_size", &CacheManager::block_size)
+      .def_property_readonly("pools", [](py::object self) {
+        auto& c = self.cast<CacheManager&>();
+        py::list out;                  // every element keeps the manager alive
+        for (auto& p : c.pools) out.append(py::cast(&p, py::return_value_policy::reference_internal, self));
+        return out;
+      })
+      .def_property_readonly("slots", [](CacheManager& c) { return &c.slots; }, py::return_value_policy::reference_internal)
+      .def("add", &CacheManager::add, py::arg("rid"))
+      .def("get", &CacheManager::get, py::arg("rid"))
+      .def("__contains__", &CacheManager::contains)
+      .def("free", &CacheManager::free)
+      .def("blocks_needed", &CacheManager::blocks_needed)
+      .def("can_grow", &CacheManager::can_grow)
+      .def("grow", &CacheManager::grow)
+      .def("commit", &CacheManager::commit)
+      .def("slot_of", &CacheManager::slot_of)
+      .def("check", &CacheManager::check)
+      .def("stats", &CacheManager::stats)
+      .def("step_shape", &CacheManager::step_shape)
+      .def("fill_step", &CacheManager::fill_step);
+
+  py::class_<DecodeRows>(m, "DecodeRows")
+      .def(py::init<std::shared_ptr<CacheManager>, int, int, std::vector<long>>())
+      .def("fill", &DecodeRows::fill)
+      .def("pad_all", &DecodeRows::pad_all);
+
+  py::class_<Request, RequestP>(m, "Request")
+      .def_readonly("rid", &Request::rid)
+      .def_readonly("prompt", &Request::prompt)
+      .def_readonly("params", &Request::params)
+      .def_readonly("seed", &Request::seed)
+      .def_readonly("arrival", &Request::arrival)
+      .def_readwrite("state", &Request::state)
+      .def_readonly("output", &Request::output)
+      .def_readwrite("num_computed", &Request::num_computed)
+      .def_readwrite("resumed", &Request::resumed)
+      .def_readwrite("finish_reason", &Request::finish_reason)
+      .def_readwrite("preemptions", &Request::preemptions)
+      .def_property_readonly("prompt_len", [](const Request& r) { return (int)r.prompt.size(); })
+      .def_property_readonly("tokens", &Request::tokens)
+      .def_property_readonly("num_tokens", &Request::num_tokens)
+      .def_property_readonly("remaining", &Request::remaining)
+      .def_property_readonly("decoding", &Request::decoding)
+      .def("token_at", &Request::token_at)
+      .def("tokens_slice", &Request::tokens_slice);
+
+  py::class_<Portion>(m, "Portion")
+      .def_readonly("request", &Portion::request)
+      .def_readonly("start", &Portion::start)
+      .def_readonly("length", &Portion::length)
+      .def_property_readonly("samples", &Portion::samples);
+
+  py::class_<StepPlan>(m, "StepPlan")
+      .def_readonly("portions", &StepPlan::portions)
+      .def_readonly("preempted", &StepPlan::preempted)
+      .def_readonly("finished", &StepPlan::finished)
+      .def_property_readonly("num_tokens", &StepPlan::num_tokens);
+
+  py::class_<Scheduler>(m, "Scheduler")
+      .def(py::init<std::shared_ptr<CacheManager>, int, int, int, py::object, std::vector<int>>(), py::arg("manager"),
+           py::kw_only(), py::arg("max_num_seqs"), py::arg("max_num_batched_tokens"), py::arg("max_model_len"),
+           py::arg("max_chunk") = py::none(), py::arg("eos_token_ids") = std::vector<int>())
+      .def_readonly("manager", &Scheduler::manager)
+      .def_readonly("max_num_seqs", &Scheduler::max_num_seqs)
+      .def_readonly("budget", &Scheduler::budget)
+      .def_readonly("max_model_len", &Scheduler::max_model_len)
+      .def_readonly("max_chunk", &Scheduler::max_chunk)
+      .def_property_readonly("waiting", [](const Scheduler& s) { return std::vector<RequestP>(s.waiting.begin(), s.waiting.end()); })
+      .def_readonly("running", &Scheduler::running)
+      .def_property_readonly("requests", [](const Scheduler& s) {
+        py::dict d;
+        for (auto& kv : s.requests) d[kv.first] = kv.second;
+        return d;
+      })
+      .def_property_readonly("num_arrivals", [](const Scheduler& s) { return s.arrivals; })
+      .def_property_readonly("counters", &Scheduler::counters)
+      .def("pool_tokens", &Scheduler::pool_tokens)
+      .def("add", &Scheduler::add, py::arg("rid"), py::arg("prompt"), py::arg("params"), py::arg("seed"))
+      .def("abort", &Scheduler::abort, py::arg("rid"))
+      .def("has_work", &Scheduler::has_work)
+      .def("schedule", &Scheduler::schedule)
+      .def("complete", &Scheduler::complete, py::arg("plan"), py::arg("sampled"));
+}

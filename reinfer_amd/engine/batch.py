@@ -15,7 +15,6 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
-import numpy as np
 import torch
 
 
@@ -55,18 +54,13 @@ class StepBatch:
 
 def build_step_batch(entries: Sequence[StepEntry], manager, device: torch.device,
                      pin: bool = False) -> StepBatch:
-    """Pack index arrays for ``entries``; the manager already holds their blocks."""
+    """Pack index arrays for ``entries``; the manager already holds their blocks.
+    The host runtime fills the buffer (CacheManager.fill_step)."""
+    entries = list(entries)
     n = len(entries)
-    bs = manager.block_size
     n_groups = len(manager.groups)
-    q_lens = [len(e.tokens) for e in entries]
+    q_lens, starts, widths, n_out = manager.step_shape(entries)
     T = sum(q_lens)
-    rcs = [manager.get(e.rid) for e in entries]
-    starts = [rc.num_tokens for rc in rcs]
-    widths = []
-    for g in range(n_groups):
-        widths.append(max(1, max(len(rc.tables[g]) for rc in rcs)))
-    n_out = sum(len(e.want) for e in entries)
 
     # layout of the packed buffer
     sizes = [T, T, T, n + 1, n, n, n, n, max(n_out, 1), T]
@@ -75,37 +69,7 @@ def build_step_batch(entries: Sequence[StepEntry], manager, device: torch.device
     for s in sizes:
         offs.append(offs[-1] + s)
     host = torch.zeros(offs[-1], dtype=torch.int32, pin_memory=pin)
-    h = host.numpy()
-    o_tok, o_pos, o_seq, o_cu, o_start, o_ctx, o_state, o_fresh, o_rows, o_noslot = offs[:10]
-    o_tab = offs[10:10 + n_groups]
-    o_slot = offs[10 + n_groups:10 + 2 * n_groups]
-
-    t = 0
-    r = 0
-    for i, (e, rc) in enumerate(zip(entries, rcs)):
-        q = q_lens[i]
-        h[o_tok + t:o_tok + t + q] = list(e.tokens)
-        h[o_pos + t:o_pos + t + q] = range(starts[i], starts[i] + q)
-        h[o_seq + t:o_seq + t + q] = i
-        h[o_cu + i] = t
-        h[o_start + i] = starts[i]
-        h[o_ctx + i] = starts[i] + q
-        h[o_state + i] = rc.slot
-        h[o_fresh + i] = 1 if rc.fresh else 0
-        for w in e.want:
-            h[o_rows + r] = t + w
-            r += 1
-        for g in range(n_groups):
-            table = rc.tables[g]
-            row = o_tab[g] + i * widths[g]
-            # entries given back (-1) are never read by a kernel; 0 keeps every index valid
-            h[row:row + len(table)] = [b if b >= 0 else 0 for b in table]
-            pos = np.arange(starts[i], starts[i] + q)
-            blk = np.asarray(table, dtype=np.int64)[pos // bs]
-            h[o_slot[g] + t:o_slot[g] + t + q] = np.where(blk < 0, -1, blk * bs + pos % bs)
-        t += q
-    h[o_cu + n] = T
-    h[o_noslot:o_noslot + T] = -1
+    manager.fill_step(entries, host.numpy(), offs[:-1], widths)
 
     dev = host.to(device, non_blocking=pin)
 
@@ -120,5 +84,5 @@ def build_step_batch(entries: Sequence[StepEntry], manager, device: torch.device
         logit_rows=view(8)[:n_out] if n_out else None, no_slots=view(9),
         block_tables=[view(10 + g, (n, widths[g])) for g in range(n_groups)],
         slots=[view(10 + n_groups + g) for g in range(n_groups)],
-        q_lens=q_lens, starts=starts, max_q_len=max(q_lens),
+        q_lens=list(q_lens), starts=list(starts), max_q_len=max(q_lens),
         max_ctx_len=max(s + q for s, q in zip(starts, q_lens)))

@@ -24,6 +24,7 @@ import numpy as np
 import torch
 
 from .. import kernels
+from .._hostlib import host as host_runtime
 from .batch import StepBatch, StepEntry
 
 MAX_GRAPH_BATCH = 64
@@ -71,19 +72,18 @@ class _CapturedStep:
             a, b = self.off[name]
             return self.dev[a:b]
 
-        self.h_seeds = hv("seeds").view(np.int64)
-        self.h_temps = hv("temps").view(np.float32)
-        self.h_tables = [hv(f"table{g}").reshape(B, W) for g in range(n_groups)]
-        self.h_slots = [hv(f"slots{g}") for g in range(n_groups)]
-        self._hv = hv
         # what never changes
         hv("seq_of_token")[:] = np.arange(B)
         hv("cu_tokens")[:] = np.arange(B + 1)
         hv("logit_rows")[:] = np.arange(B)
         hv("no_slots")[:] = -1
-        self.row_owner: List[Optional[object]] = [None] * B
-        self.row_len = [[0] * B for _ in range(n_groups)]
-        self._pad_rows(0, B)
+        # the host runtime keeps track of which request sits in which row and writes what changed
+        order = ["token_ids", "positions", "start_pos", "ctx_lens", "state_slots", "fresh", "sample_pos",
+                 "temps", "seeds"]
+        for g in range(n_groups):
+            order += [f"table{g}", f"slots{g}"]
+        self.rows = host_runtime.DecodeRows(runner.manager, B, W, [self.off[k][0] for k in order])
+        self.rows.pad_all(self.h)
 
         self.seeds = dv("seeds").view(torch.int64)
         self.temps = dv("temps").view(torch.float32)
@@ -106,17 +106,6 @@ class _CapturedStep:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self._capture(pool)
 
-    def _pad_rows(self, lo: int, hi: int) -> None:
-        hv = self._hv
-        for name, val in (("token_ids", 0), ("positions", 0), ("start_pos", 0), ("ctx_lens", 1),
-                          ("state_slots", -1), ("fresh", 0), ("sample_pos", 0), ("temps", 0)):
-            hv(name)[lo:hi] = val
-        self.h_seeds[lo:hi] = 0
-        for g, s in enumerate(self.h_slots):
-            s[lo:hi] = -1
-        for i in range(lo, hi):
-            self.row_owner[i] = None
-
     def _body(self) -> None:
         r = self.runner
         self.logits = r.model.forward(self.batch, r.caches)
@@ -136,42 +125,8 @@ class _CapturedStep:
         with torch.cuda.graph(self.graph, pool=pool), torch.no_grad():
             self._body()
 
-    def fill(self, entries: Sequence[StepEntry], rcs, sampling) -> None:
-        bs = self.runner.block_size
-        hv = self._hv
-        tok, pos, start, ctx = hv("token_ids"), hv("positions"), hv("start_pos"), hv("ctx_lens")
-        state, fresh, spos = hv("state_slots"), hv("fresh"), hv("sample_pos")
-        n = len(entries)
-        for i, (e, rc) in enumerate(zip(entries, rcs)):
-            p = rc.num_tokens
-            tok[i] = e.tokens[0]
-            pos[i] = p
-            start[i] = p
-            ctx[i] = p + 1
-            state[i] = rc.slot
-            fresh[i] = 1 if rc.fresh else 0
-            same = self.row_owner[i] is rc
-            for g, table in enumerate(rc.tables):
-                have = self.row_len[g][i] if same else 0
-                if len(table) > have:
-                    # entries given back (-1) are never read; 0 keeps every index valid
-                    self.h_tables[g][i, have:len(table)] = [b if b >= 0 else 0 for b in table[have:]]
-                self.row_len[g][i] = len(table)
-                blk = table[p // bs]
-                self.h_slots[g][i] = -1 if blk < 0 else blk * bs + p % bs
-            self.row_owner[i] = rc
-        if sampling is not None:
-            temps, seeds, positions = sampling
-            self.h_temps[:n] = temps
-            self.h_seeds[:n] = seeds
-            spos[:n] = positions
-        else:
-            self.h_temps[:n] = 0.0
-            self.h_seeds[:n] = 0
-            spos[:n] = 0
-        hi = max(i for i, o in enumerate(self.row_owner) if o is not None) + 1
-        if hi > n:
-            self._pad_rows(n, hi)
+    def fill(self, entries: Sequence[StepEntry], sampling) -> None:
+        self.rows.fill(list(entries), self.h, sampling)
 
     def replay(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
@@ -206,7 +161,7 @@ class DecodeGraphs:
                 self.pool = torch.cuda.graph_pool_handle()
             cs = _CapturedStep(r, B, ctx_cap, self.pool)
             self.steps[key] = cs
-        cs.fill(entries, rcs, sampling)
+        cs.fill(entries, sampling)
         cs.replay()
         self.replays += 1
         return cs.logits, cs.tokens

@@ -75,9 +75,9 @@ class LLMEngine:
         for t in prompt_token_ids:
             if not 0 <= int(t) < V:
                 raise RequestRefused(f"token {t} outside the vocabulary of {V}")
-        arrival = self.scheduler._arrivals
+        arrival = self.scheduler.num_arrivals
         seed = params.seed if params.seed is not None else derive_seed(self.seed, arrival)
-        self.scheduler.add(rid, prompt_token_ids, params, seed)
+        self.scheduler.add(rid, [int(t) for t in prompt_token_ids], params, seed)
         return rid
 
     def abort(self, rid: Hashable) -> bool:
@@ -98,11 +98,7 @@ class LLMEngine:
         entries, rows = [], []
         for p in plan.portions:
             r = p.request
-            if p.length == 1:
-                i = p.start
-                toks = [r.prompt[i] if i < len(r.prompt) else r.output[i - len(r.prompt)]]
-            else:
-                toks = r.tokens[p.start:p.start + p.length]
+            toks = r.tokens_slice(p.start, p.length)
             entries.append(StepEntry(r.rid, toks, [p.length - 1] if p.samples else []))
             if p.samples:
                 rows.append(r)
