@@ -26,6 +26,11 @@ class RequestRefused(ValueError):
     pass
 
 
+class StepError(ValueError):
+    """A step was asked for something it cannot run (checked before any launch);
+    the reference's step checks the same on the host (crates/cuda/src/engine.rs:5854-5943)."""
+
+
 def _load():
     name = "reinfer_amd._host"
     if name in sys.modules:
@@ -35,7 +40,7 @@ def _load():
     spec = importlib.util.spec_from_file_location(name, path)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    mod.set_exceptions(OutOfBlocks, OutOfSlots, RequestRefused)
+    mod.set_exceptions(OutOfBlocks, OutOfSlots, RequestRefused, StepError)
     sys.modules[name] = mod
     return mod
 

@@ -40,6 +40,7 @@ namespace py = pybind11;
 static py::object* E_OutOfBlocks = nullptr;
 static py::object* E_OutOfSlots = nullptr;
 static py::object* E_RequestRefused = nullptr;
+static py::object* E_StepError = nullptr;
 
 [[noreturn]] static void raise_instance(const py::object& cls, const py::object& inst) {
   PyErr_SetObject(cls.ptr(), inst.ptr());
@@ -47,6 +48,9 @@ static py::object* E_RequestRefused = nullptr;
 }
 [[noreturn]] static void out_of_blocks(int group, int need, int free_) {
   raise_instance(*E_OutOfBlocks, (*E_OutOfBlocks)(group, need, free_));
+}
+[[noreturn]] static void step_error(const std::string& msg) {
+  raise_instance(*E_StepError, (*E_StepError)(msg));
 }
 [[noreturn]] static void assertion(const std::string& msg) {
   PyErr_SetString(PyExc_AssertionError, msg.c_str());
@@ -122,6 +126,15 @@ struct SlotPool {
     free_.push_back(s);
   }
 };
+
+// A request's part in a step: its next tokens and where logits are wanted (indices into tokens).
+struct StepEntry {
+  py::object rid;
+  std::vector<int> tokens;
+  std::vector<int> want;
+};
+using StepEntryP = std::shared_ptr<StepEntry>;
+using StepEntries = std::vector<StepEntryP>;
 
 // ------------------------------------------------------------------ manager
 struct RequestCache {
@@ -316,14 +329,14 @@ struct CacheManager {
   // ------------------------------------------------------ a step's index arrays
   // Sizes of the packed int32 buffer of a step over `entries` (objects with rid, tokens, want):
   // -> (q_lens, starts, widths per group, wanted rows). The layout itself is the caller's.
-  py::tuple step_shape(const py::list& entries) const {
+  py::tuple step_shape(const StepEntries& entries) const {
     std::vector<int> q_lens, starts, widths(n_groups(), 1);
     int n_out = 0;
-    for (auto e : entries) {
-      auto rc = get(e.attr("rid").cast<py::object>());
-      q_lens.push_back((int)py::len(e.attr("tokens")));
+    for (auto& e : entries) {
+      auto rc = get(e->rid);
+      q_lens.push_back((int)e->tokens.size());
       starts.push_back(rc->num_tokens);
-      n_out += (int)py::len(e.attr("want"));
+      n_out += (int)e->want.size();
       for (int g = 0; g < n_groups(); ++g) widths[g] = std::max(widths[g], (int)rc->tables[g].size());
     }
     return py::make_tuple(q_lens, starts, widths, n_out);
@@ -333,48 +346,95 @@ struct CacheManager {
   // token, first token of each request (n + 1), start, context length, state slot, fresh flag,
   // wanted rows, "store nothing" slots, then per group the block tables [n, width] and after all
   // tables per group the cache slot of each token.
-  void fill_step(const py::list& entries, py::array_t<int32_t, py::array::c_style> buffer,
+  void fill_step(const StepEntries& entries, py::array_t<int32_t, py::array::c_style> buffer,
                  const std::vector<long>& offs, const std::vector<int>& widths) const {
-    auto h = buffer.mutable_unchecked<1>();
-    const int n = (int)py::len(entries), G = n_groups();
+    int32_t* h = buffer.mutable_data();
+    const int n = (int)entries.size(), G = n_groups();
     if ((int)offs.size() != 10 + 2 * G || (int)widths.size() != G) throw py::value_error("fill_step: bad layout");
     const long o_tok = offs[0], o_pos = offs[1], o_seq = offs[2], o_cu = offs[3], o_start = offs[4], o_ctx = offs[5],
                o_state = offs[6], o_fresh = offs[7], o_rows = offs[8], o_noslot = offs[9];
     long t = 0, r = 0;
-    int i = 0;
-    for (auto e : entries) {
-      auto rc = get(e.attr("rid").cast<py::object>());
-      const int start = rc->num_tokens;
-      int q = 0;
-      for (auto tok : e.attr("tokens")) {
-        h(o_tok + t + q) = tok.cast<int32_t>();
-        h(o_pos + t + q) = start + q;
-        h(o_seq + t + q) = i;
-        h(o_noslot + t + q) = -1;
-        ++q;
+    for (int i = 0; i < n; ++i) {
+      const StepEntry& e = *entries[i];
+      auto rc = get(e.rid);
+      const int start = rc->num_tokens, q = (int)e.tokens.size();
+      for (int j = 0; j < q; ++j) {
+        h[o_tok + t + j] = e.tokens[j];
+        h[o_pos + t + j] = start + j;
+        h[o_seq + t + j] = i;
+        h[o_noslot + t + j] = -1;
       }
-      h(o_cu + i) = (int32_t)t;
-      h(o_start + i) = start;
-      h(o_ctx + i) = start + q;
-      h(o_state + i) = rc->slot;
-      h(o_fresh + i) = rc->fresh ? 1 : 0;
-      for (auto w : e.attr("want")) h(o_rows + r++) = (int32_t)(t + w.cast<int>());
+      h[o_cu + i] = (int32_t)t;
+      h[o_start + i] = start;
+      h[o_ctx + i] = start + q;
+      h[o_state + i] = rc->slot;
+      h[o_fresh + i] = rc->fresh ? 1 : 0;
+      for (int w : e.want) h[o_rows + r++] = (int32_t)(t + w);
       for (int g = 0; g < G; ++g) {
         const auto& table = rc->tables[g];
         const long row = offs[10 + g] + (long)i * widths[g];
         // entries given back (-1) are never read by a kernel; 0 keeps every index valid
-        for (size_t b = 0; b < table.size(); ++b) h(row + (long)b) = table[b] >= 0 ? table[b] : 0;
+        for (size_t b = 0; b < table.size(); ++b) h[row + (long)b] = table[b] >= 0 ? table[b] : 0;
         const long o_slot = offs[10 + G + g];
         for (int j = 0; j < q; ++j) {
           const int pos = start + j;
           const int blk = table.at(pos / block_size);
-          h(o_slot + t + j) = blk < 0 ? -1 : blk * block_size + pos % block_size;
+          h[o_slot + t + j] = blk < 0 ? -1 : blk * block_size + pos % block_size;
         }
       }
       t += q;
-      ++i;
     }
-    h(o_cu + n) = (int32_t)t;
+    h[o_cu + n] = (int32_t)t;
+  }
+
+  // Before a step: check the entries (the reference's step checks the same on the host,
+  // crates/cuda/src/engine.rs:5854-5943), then take the blocks their tokens need, all or none.
+  // -> (every entry brings one token, every entry wants one row, the longest context after the step)
+  py::tuple begin_step(const StepEntries& entries, int vocab, int max_model_len) {
+    bool one_token = true, one_want = true;
+    int longest = 0;
+    if (entries.empty()) step_error("a step needs at least one request");
+    std::vector<RequestCache*> rcs;
+    const int G = n_groups();
+    std::vector<int> total(G, 0), need(G);
+    for (size_t i = 0; i < entries.size(); ++i) {
+      const StepEntry& e = *entries[i];
+      for (size_t k = 0; k < i; ++k)
+        if (entries[k]->rid.equal(e.rid)) step_error("request " + show(e.rid) + " appears twice in one step");
+      auto it = requests.find(e.rid);
+      if (it == requests.end()) step_error("request " + show(e.rid) + " is not live");
+      if (e.tokens.empty()) step_error("request " + show(e.rid) + " brings no tokens");
+      for (int tok : e.tokens)
+        if (tok < 0 || tok >= vocab)
+          step_error("request " + show(e.rid) + ": token " + std::to_string(tok) + " outside the vocabulary of " + std::to_string(vocab));
+      for (int w : e.want)
+        if (w < 0 || w >= (int)e.tokens.size())
+          step_error("request " + show(e.rid) + ": logits wanted at " + std::to_string(w) + " of " + std::to_string(e.tokens.size()) + " tokens");
+      RequestCache* rc = it->second.get();
+      const int new_total = rc->num_tokens + (int)e.tokens.size();
+      if (new_total > max_model_len)
+        step_error("request " + show(e.rid) + ": " + std::to_string(new_total) + " tokens exceed the context of " + std::to_string(max_model_len));
+      blocks_needed_into(*rc, new_total, need.data());
+      for (int g = 0; g < G; ++g) total[g] += need[g];
+      rcs.push_back(rc);
+      one_token = one_token && e.tokens.size() == 1;
+      one_want = one_want && e.want.size() == 1;
+      longest = std::max(longest, new_total);
+    }
+    int worst = -1;
+    for (int g = 0; g < G; ++g)
+      if (total[g] > pools[g].num_free() && (worst < 0 || total[g] - pools[g].num_free() > total[worst] - pools[worst].num_free()))
+        worst = g;
+    if (worst >= 0) out_of_blocks(worst, total[worst], pools[worst].num_free());
+    for (size_t i = 0; i < entries.size(); ++i) grow_rc(*rcs[i], rcs[i]->num_tokens + (int)entries[i]->tokens.size());
+    return py::make_tuple(one_token, one_want, longest);
+  }
+  // After the step: its tokens are stored.
+  void end_step(const StepEntries& entries) {
+    for (auto& e : entries) {
+      auto rc = get(e->rid);
+      commit_rc(*rc, rc->num_tokens + (int)e->tokens.size());
+    }
   }
 };
 
@@ -414,15 +474,17 @@ struct DecodeRows {
   }
 
   // entries: objects with rid and tokens (one each); sampling: None or (temperatures, seeds, positions)
-  void fill(const py::list& entries, py::array_t<int32_t, py::array::c_style> buffer, const py::object& sampling) {
+  // The entries' blocks are already taken (begin_step): a token's position is the request's length before
+  // the step.
+  void fill(const StepEntries& entries, py::array_t<int32_t, py::array::c_style> buffer, const py::object& sampling) {
     int32_t* h = buffer.mutable_data();
-    const int n = (int)py::len(entries), G = manager->n_groups(), bs = manager->block_size;
+    const int n = (int)entries.size(), G = manager->n_groups(), bs = manager->block_size;
     if (n > B) throw py::value_error("DecodeRows: more entries than rows");
-    int i = 0;
-    for (auto e : entries) {
-      auto rc = manager->get(e.attr("rid").cast<py::object>());
+    for (int i = 0; i < n; ++i) {
+      const StepEntry& e = *entries[i];
+      auto rc = manager->get(e.rid);
       const int p = rc->num_tokens;
-      h[offs[0] + i] = (*e.attr("tokens").begin()).cast<int32_t>();
+      h[offs[0] + i] = e.tokens.at(0);
       h[offs[1] + i] = p;
       h[offs[2] + i] = p;
       h[offs[3] + i] = p + 1;
@@ -441,7 +503,6 @@ struct DecodeRows {
         h[offs[9 + 2 * g + 1] + i] = blk < 0 ? -1 : blk * bs + p % bs;
       }
       owner[i] = rc->serial;
-      ++i;
     }
     if (!sampling.is_none()) {
       auto s = sampling.cast<py::tuple>();
@@ -496,6 +557,9 @@ struct Request {
   // read once from params
   int max_tokens = 0;
   bool ignore_eos = false;
+  bool filters = false;            // anything beside temperature shapes the distribution
+  float temperature = 0.f;
+  int64_t seed64 = 0;              // the seed's low 64 bits as the kernels take them
   std::vector<int> stop_ids;
 
   int num_tokens() const { return (int)(prompt.size() + output.size()); }
@@ -581,9 +645,15 @@ struct Scheduler {
     req->prompt = prompt;
     req->params = params;
     req->seed = seed;
+    {
+      py::int_ mask((uint64_t)0xFFFFFFFFFFFFFFFFull);
+      req->seed64 = (int64_t)py::reinterpret_steal<py::int_>(PyNumber_And(seed.ptr(), mask.ptr())).cast<uint64_t>();
+    }
     req->arrival = arrivals++;
     req->max_tokens = params.attr("max_tokens").cast<int>();
     req->ignore_eos = params.attr("ignore_eos").cast<bool>();
+    req->filters = params.attr("filters").cast<bool>();
+    req->temperature = std::max(0.f, params.attr("temperature").cast<float>());
     for (auto t : params.attr("stop_token_ids")) req->stop_ids.push_back(t.cast<int>());
     requests[rid] = req;
     waiting.push_back(req);
@@ -731,13 +801,22 @@ struct Scheduler {
   // stop ids, then the cap on new tokens, then the context (crates/scheduler/src/req.rs:281-314);
   // the stop token is consumed, not emitted.
   std::vector<RequestP> complete(const StepPlan& plan, const py::dict& sampled) {
+    std::vector<int> tokens;
+    for (auto& p : plan.portions)
+      if (p.samples()) tokens.push_back(sampled[p.request->rid].cast<int>());
+    return complete_tokens(plan, tokens);
+  }
+  // The same with the sampled tokens as a list in the order of the portions that sample.
+  std::vector<RequestP> complete_tokens(const StepPlan& plan, const std::vector<int>& tokens) {
     std::vector<RequestP> done;
+    size_t next = 0;
     for (auto& p : plan.portions) {
       auto& r = p.request;
       const bool samples = p.samples();        // before the cursor and the output move
       r->num_computed = p.start + p.length;
       if (!samples) continue;
-      const int tok = sampled[r->rid].cast<int>();
+      if (next >= tokens.size()) throw py::value_error("complete: fewer tokens than portions that sample");
+      const int tok = tokens[next++];
       const bool is_eos = std::find(eos.begin(), eos.end(), tok) != eos.end();
       const bool stop = (is_eos && !r->ignore_eos) ||
                         std::find(r->stop_ids.begin(), r->stop_ids.end(), tok) != r->stop_ids.end();
@@ -759,6 +838,39 @@ struct Scheduler {
     return done;
   }
 
+  // The plan as the step function takes it: one entry per portion, logits wanted at a portion's last
+  // token where it reaches the request's end. -> (entries, requests that sample in entry order,
+  // (temperatures, seeds, positions) if every entry samples and none uses filters, else None)
+  py::tuple entries_for(const StepPlan& plan) const {
+    StepEntries entries;
+    std::vector<RequestP> rows;
+    bool plain = true;
+    for (auto& p : plan.portions) {
+      auto e = std::make_shared<StepEntry>();
+      e->rid = p.request->rid;
+      e->tokens = p.request->tokens_slice(p.start, p.length);
+      if (p.samples()) {
+        e->want.push_back(p.length - 1);
+        rows.push_back(p.request);
+        plain = plain && !p.request->filters;
+      } else {
+        plain = false;
+      }
+      entries.push_back(std::move(e));
+    }
+    py::object sampling = py::none();
+    if (plain && !rows.empty()) {
+      py::list temps, seeds, positions;
+      for (auto& r : rows) {
+        temps.append(r->temperature);
+        seeds.append(r->seed64);
+        positions.append(r->num_tokens());
+      }
+      sampling = py::make_tuple(temps, seeds, positions);
+    }
+    return py::make_tuple(entries, rows, sampling);
+  }
+
   py::dict counters() const {
     py::dict d;
     d["steps"] = c_steps;
@@ -772,11 +884,30 @@ struct Scheduler {
 
 PYBIND11_MODULE(_host, m) {
   m.doc() = "host runtime of reinfer_amd: cache bookkeeping, step packing, scheduler";
-  m.def("set_exceptions", [](py::object oob, py::object oos, py::object refused) {
+  m.def("set_exceptions", [](py::object oob, py::object oos, py::object refused, py::object step) {
     E_OutOfBlocks = new py::object(std::move(oob));
     E_OutOfSlots = new py::object(std::move(oos));
     E_RequestRefused = new py::object(std::move(refused));
+    E_StepError = new py::object(std::move(step));
   });
+
+  py::class_<StepEntry, StepEntryP>(m, "StepEntry", "A request's part in a step: its next tokens and where logits are wanted.")
+      .def(py::init([](py::object rid, std::vector<int> tokens, std::vector<int> want) {
+             auto e = std::make_shared<StepEntry>();
+             e->rid = std::move(rid);
+             e->tokens = std::move(tokens);
+             e->want = std::move(want);
+             return e;
+           }),
+           py::arg("rid"), py::arg("tokens"), py::arg("want") = std::vector<int>())
+      .def_readonly("rid", &StepEntry::rid)
+      .def_readonly("tokens", &StepEntry::tokens)
+      .def_readonly("want", &StepEntry::want)
+      .def_property_readonly("num_tokens", [](const StepEntry& e) { return e.tokens.size(); })
+      .def("__repr__", [](const StepEntry& e) {
+        return "StepEntry(" + show(e.rid) + ", " + std::to_string(e.tokens.size()) + " tokens, " +
+               std::to_string(e.want.size()) + " wanted)";
+      });
   m.attr("WAITING") = WAITING;
   m.attr("RUNNING") = RUNNING;
   m.attr("FINISHED") = FINISHED;
@@ -831,7 +962,9 @@ PYBIND11_MODULE(_host, m) {
       .def("check", &CacheManager::check)
       .def("stats", &CacheManager::stats)
       .def("step_shape", &CacheManager::step_shape)
-      .def("fill_step", &CacheManager::fill_step);
+      .def("fill_step", &CacheManager::fill_step)
+      .def("begin_step", &CacheManager::begin_step, py::arg("entries"), py::arg("vocab"), py::arg("max_model_len"))
+      .def("end_step", &CacheManager::end_step, py::arg("entries"));
 
   py::class_<DecodeRows>(m, "DecodeRows")
       .def(py::init<std::shared_ptr<CacheManager>, int, int, std::vector<long>>())
@@ -893,5 +1026,7 @@ PYBIND11_MODULE(_host, m) {
       .def("abort", &Scheduler::abort, py::arg("rid"))
       .def("has_work", &Scheduler::has_work)
       .def("schedule", &Scheduler::schedule)
-      .def("complete", &Scheduler::complete, py::arg("plan"), py::arg("sampled"));
+      .def("entries_for", &Scheduler::entries_for, py::arg("plan"))
+      .def("complete", &Scheduler::complete, py::arg("plan"), py::arg("sampled"))
+      .def("complete_tokens", &Scheduler::complete_tokens, py::arg("plan"), py::arg("tokens"));
 }

@@ -13,17 +13,16 @@ The reference has two separate calls instead, a whole prompt from position 0
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, List, Optional, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
+from .._hostlib import host as _host
 
-@dataclass
-class StepEntry:
-    """A request's part in a step: its next tokens and where logits are wanted."""
-    rid: Hashable
-    tokens: Sequence[int]
-    want: Sequence[int] = ()        # indices into ``tokens``
+# A request's part in a step, ``StepEntry(rid, tokens, want=[])``: its next tokens and the
+# indices into them where logits are wanted. Kept by the host runtime so that checking,
+# block growth and packing read it without a call back into Python.
+StepEntry = _host.StepEntry
 
 
 @dataclass

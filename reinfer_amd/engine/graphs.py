@@ -125,8 +125,8 @@ class _CapturedStep:
         with torch.cuda.graph(self.graph, pool=pool), torch.no_grad():
             self._body()
 
-    def fill(self, entries: Sequence[StepEntry], sampling) -> None:
-        self.rows.fill(list(entries), self.h, sampling)
+    def fill(self, entries: List[StepEntry], sampling) -> None:
+        self.rows.fill(entries, self.h, sampling)
 
     def replay(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
@@ -140,18 +140,12 @@ class DecodeGraphs:
         self.pool = None
         self.replays = 0
 
-    def eligible(self, entries: Sequence[StepEntry]) -> bool:
-        if len(entries) > MAX_GRAPH_BATCH:
-            return False
-        return all(len(e.tokens) == 1 for e in entries)
-
-    def run(self, entries: Sequence[StepEntry], sampling=None):
-        """-> (logits [B_pad, vocab] static, tokens [B_pad] static): rows past the
+    def run(self, entries: List[StepEntry], longest: int, sampling=None):
+        """A step of at most MAX_GRAPH_BATCH entries with one token each; ``longest`` is the longest
+        context after it. -> (logits [B_pad, vocab] static, tokens [B_pad] static): rows past the
         entries are padding; both are overwritten by the next replay of this bucket."""
         r = self.runner
-        rcs = [r.manager.get(e.rid) for e in entries]
         B = _bucket(len(entries))
-        longest = max(rc.num_tokens for rc in rcs) + 1
         ctx_cap = max(256, _bucket(longest))
         ctx_cap = min(ctx_cap, max(256, _bucket(r.max_model_len)))
         key = (B, ctx_cap)

@@ -21,7 +21,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 import torch
 
 from ..config import load_config
-from ..sampling import Sampler, SamplingError, SamplingParams, as_int64, derive_seed
+from ..sampling import Sampler, SamplingError, SamplingParams, derive_seed
 from .batch import StepEntry
 from .runner import ModelRunner
 from .scheduler import FINISHED, Request, RequestRefused, Scheduler, StepPlan
@@ -95,33 +95,21 @@ class LLMEngine:
             if not finished and self.scheduler.has_work() and not plan.preempted:
                 raise RuntimeError("the scheduler could place no token although work is waiting")
             return finished
-        entries, rows = [], []
-        for p in plan.portions:
-            r = p.request
-            toks = r.tokens_slice(p.start, p.length)
-            entries.append(StepEntry(r.rid, toks, [p.length - 1] if p.samples else []))
-            if p.samples:
-                rows.append(r)
-        sampled: Dict[Hashable, int] = {}
-        plain = len(rows) == len(entries) and not any(r.params.filters for r in rows)
-        if plain:
-            # every entry wants one token and none shapes its distribution: the step may draw them itself
-            sampling = ([max(0.0, float(r.params.temperature)) for r in rows],
-                        [as_int64(r.seed) for r in rows], [r.num_tokens for r in rows])
-            logits, toks = self.runner.step_sampled(entries, sampling)
-        else:
-            logits, toks = self.runner.step(entries), None
+        # entries as the step takes them; where every entry wants one token and none shapes its
+        # distribution, the step may draw the tokens itself
+        entries, rows, sampling = self.scheduler.entries_for(plan)
+        logits, toks = self.runner.step_sampled(entries, sampling)
         if toks is not None:
             out = toks.tolist()
-            for r, t in zip(rows, out):
-                if t < 0:
-                    raise SamplingError(f"request {r.rid!r}: no finite logit to sample from")
-                sampled[r.rid] = t
+            if min(out) < 0:
+                r = rows[[t < 0 for t in out].index(True)]
+                raise SamplingError(f"request {r.rid!r}: no finite logit to sample from")
         elif rows:
             out = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
                                       [r.num_tokens for r in rows], [r.tokens for r in rows])
-            sampled = {r.rid: t for r, t in zip(rows, out)}
-        done = self.scheduler.complete(plan, sampled)
+        else:
+            out = []
+        done = self.scheduler.complete_tokens(plan, out)
         return finished + [self._output(r) for r in done]
 
     @staticmethod

@@ -19,15 +19,12 @@ from ..config.schema import ModelSpec
 from ..models import DecoderModel, declare_params
 from ..parts import KVNeed, LayerCache, StateNeed
 from ..weights import check_tensors, load_weights, random_tensors, storage_dtype
+from .._hostlib import StepError
 from .batch import StepBatch, StepEntry, build_step_batch
+from .graphs import MAX_GRAPH_BATCH
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
            "fp32": torch.float32, "f32": torch.float32}
-
-
-class StepError(ValueError):
-    """A step was asked for something it cannot run (checked before any launch);
-    the reference's step checks the same on the host (crates/cuda/src/engine.rs:5854-5943)."""
 
 
 def parse_dtype(dtype) -> torch.dtype:
@@ -170,29 +167,6 @@ class ModelRunner:
         return self.manager.get(rid).num_tokens
 
     # --------------------------------------------------------------- step
-    def check_entries(self, entries: Sequence[StepEntry]) -> None:
-        if not entries:
-            raise StepError("a step needs at least one request")
-        seen = set()
-        V = self.spec.vocab_size
-        for e in entries:
-            if e.rid in seen:
-                raise StepError(f"request {e.rid!r} appears twice in one step")
-            seen.add(e.rid)
-            if e.rid not in self.manager:
-                raise StepError(f"request {e.rid!r} is not live")
-            if len(e.tokens) == 0:
-                raise StepError(f"request {e.rid!r} brings no tokens")
-            for tok in e.tokens:
-                if not 0 <= int(tok) < V:
-                    raise StepError(f"request {e.rid!r}: token {tok} outside the vocabulary of {V}")
-            for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise StepError(f"request {e.rid!r}: logits wanted at {w} of {len(e.tokens)} tokens")
-            total = self.manager.get(e.rid).num_tokens + len(e.tokens)
-            if total > self.max_model_len:
-                raise StepError(f"request {e.rid!r}: {total} tokens exceed the context of {self.max_model_len}")
-
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the entries' tokens as one batch; logits [wanted, vocab] float32,
         in the order of the entries and of each entry's ``want``. The result may be
@@ -204,20 +178,16 @@ class ModelRunner:
         asks for a token from each entry's single wanted row where the step can draw it
         itself. -> (logits, tokens): ``tokens`` is an int32 device tensor, one per
         entry, or None when the caller has to sample from the logits."""
-        self.check_entries(entries)
-        growth = [(e.rid, self.manager.get(e.rid).num_tokens + len(e.tokens)) for e in entries]
-        if not self.manager.can_grow(growth):
-            need = [sum(self.manager.blocks_needed(r, t)[g] for r, t in growth)
-                    for g in range(len(self.groups))]
-            g = max(range(len(self.groups)), key=lambda i: need[i] - self.manager.pools[i].num_free)
-            raise OutOfBlocks(g, need[g], self.manager.pools[g].num_free)
-        for rid, total in growth:
-            self.manager.grow(rid, total)
+        if not isinstance(entries, list):
+            entries = list(entries)
+        # checks every entry (StepError), then takes the blocks of all of them or raises OutOfBlocks
+        one_token, one_want, longest = self.manager.begin_step(entries, self.spec.vocab_size,
+                                                               self.max_model_len)
         tokens = None
-        if self.graphs is not None and self.graphs.eligible(entries):
-            all_logits, all_tokens = self.graphs.run(entries, sampling)
+        if self.graphs is not None and one_token and len(entries) <= MAX_GRAPH_BATCH:
+            all_logits, all_tokens = self.graphs.run(entries, longest, sampling)
             n = len(entries)
-            if all(len(e.want) == 1 for e in entries):
+            if one_want:
                 logits = all_logits[:n]
                 if sampling is not None:
                     tokens = all_tokens[:n]
@@ -228,8 +198,7 @@ class ModelRunner:
         else:
             batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
             logits = self.forward(batch)
-        for rid, total in growth:
-            self.manager.commit(rid, total)
+        self.manager.end_step(entries)
         return logits, tokens
 
     def forward(self, batch: StepBatch) -> torch.Tensor:
