@@ -16,6 +16,12 @@
 // 4g + s of the first 16 keys for s < 4, of the second 16 for s >= 4, for both
 // operands alike).
 //
+// The grid is a fixed number of workgroups, as many as the chip holds at once; the
+// (token, chunk, KV head) items are numbered on the device from the tokens'
+// positions and workgroup w takes items w, w + grid, ...: launching one
+// workgroup an item costs 13 to 20 ns each (a step of 64 requests has ten
+// thousand) and leaves the last round of workgroups half empty.
+//
 // Chunks of one (token, head) are merged by a second small kernel, always in
 // chunk order. (Merging in the last workgroup to arrive needs device-wide
 // release/acquire fences in every workgroup; on this chip each one writes back
@@ -31,186 +37,237 @@
 
 #define FD_THREADS 256
 #define FD_WAVES 4
+#define FD_MAX_TOKENS 1024      // tokens of one launch; the entry point cuts longer lists
 
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int DMAX>
-__global__ void __launch_bounds__(FD_THREADS)
+__global__ void __launch_bounds__(FD_THREADS, DMAX <= 128 ? 3 : 1)
 flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                     const int* __restrict__ block_tables, int max_blocks,
                     const int* __restrict__ token_list, const int* __restrict__ seq_of_token,
                     const int* __restrict__ positions, int block_size, int Hkv, int G, int d,
-                    float scale_log2, int window, int chunk, int max_chunks,
-                    float* __restrict__ part_o, float* __restrict__ part_ml) {
+                    float scale_log2, int window, int chunk, int max_chunks, int n_tokens,
+                    int t_base, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   extern __shared__ float lds[];       // [waves][G][d] outputs, then [waves][G][2] maximum and sum
 
-  const int ci = blockIdx.x, kvh = blockIdx.y, li = blockIdx.z;
-  const int t = token_list ? token_list[li] : li;
-  const int p = positions[t];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int c_first = lo / chunk, c_last = p / chunk;
-  if (ci < c_first || ci > c_last) return;       // no key of this token in the chunk
-  const int n_chunks = c_last - c_first + 1;
-  const int seq = seq_of_token[t];
-  const int* table = block_tables + (size_t)seq * max_blocks;
+  __shared__ int first_item[FD_MAX_TOKENS + 1];   // chunks of the tokens before token i
 
   const int tid = threadIdx.x;
   const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
   const int r = lane & 15, g = lane >> 4;
-  const int Hq = Hkv * G;
 
-  // second operand of the score product: column r is query head r of the group
-  bf16x8_t qreg[NDT];
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt) {
-    const int e = dt * 32 + g * 8;
-    qreg[dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
-    if (r < G && e < d) qreg[dt] = *(const bf16x8_t*)(q + (size_t)t * q_stride + (size_t)(kvh * G + r) * d + e);
+  // every workgroup numbers the items alike: chunks of each token, then a running sum
+  for (int i = tid; i < n_tokens; i += FD_THREADS) {
+    const int pi = positions[token_list ? token_list[i] : t_base + i];
+    const int loi = (window > 0 && pi - window + 1 > 0) ? pi - window + 1 : 0;
+    first_item[i + 1] = pi / chunk - loi / chunk + 1;
   }
-  f32x4_t acc[NOT];
+  if (tid == 0) first_item[0] = 0;
+  __syncthreads();
+  if (wave == 0) {
+    const int per = (n_tokens + RA_WAVE - 1) / RA_WAVE;
+    const int b = lane * per;
+    int sum = 0;
+    for (int j = 0; j < per; ++j)
+      if (b + j < n_tokens) sum += first_item[b + j + 1];
+    int incl = sum;
 #pragma unroll
-  for (int i = 0; i < NOT; ++i) acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+    for (int o = 1; o < RA_WAVE; o <<= 1) {
+      const int up = __shfl_up(incl, o, RA_WAVE);
+      if (lane >= o) incl += up;
+    }
+    int run = incl - sum;
+    for (int j = 0; j < per; ++j)
+      if (b + j < n_tokens) {
+        run += first_item[b + j + 1];
+        first_item[b + j + 1] = run;
+      }
+  }
+  __syncthreads();
+  const int n_items = first_item[n_tokens] * Hkv;
 
-  const int k_begin = ci * chunk;
-  const int k_end = min(k_begin + chunk, p + 1);
-  for (int k0 = k_begin + wave * 32; k0 < k_end; k0 += FD_WAVES * 32) {
-    if (k0 + 31 < lo) continue;
-    // the two 16-key tiles of this step; a tile past the last key is not touched
-    bool live[2], edge[2];
-    const bf16_t* kb[2];
-    const bf16_t* vb[2];
+  int li = 0;                                     // items of a workgroup ascend: the token only moves forward
+  for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+    const int slot = item / Hkv, kvh = item % Hkv;  // KV heads of one (token, chunk) are neighbours in memory
+    while (first_item[li + 1] <= slot) ++li;
+    const int t = token_list ? token_list[li] : t_base + li;
+    const int p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int c_first = lo / chunk, c_last = p / chunk;
+    const int ci = c_first + (slot - first_item[li]);
+    const int n_chunks = c_last - c_first + 1;
+    const int seq = seq_of_token[t];
+    const int* table = block_tables + (size_t)seq * max_blocks;
+    const int Hq = Hkv * G;
+
+    // second operand of the score product: column r is query head r of the group
+    bf16x8_t qreg[NDT];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int kt = k0 + tt * 16;
-      live[tt] = kt <= p && kt + 15 >= lo;
-      edge[tt] = kt + 15 > p || kt < lo;
-      const int blk = live[tt] ? table[kt / block_size] : 0;
-      const size_t tile = ((size_t)blk * Hkv + kvh) * block_size * d + (size_t)((kt % block_size) >> 4) * 16 * d;
-      kb[tt] = kcache + tile + (g * 16 + r) * 8;        // chunk 4 dt + g of slot r
-      vb[tt] = vcache + tile + (g * 16 + r) * 4;        // slots 4g..4g+3 of row 16 ot + r
+    for (int dt = 0; dt < NDT; ++dt) {
+      const int e = dt * 32 + g * 8;
+      qreg[dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+      if (r < G && e < d) qreg[dt] = *(const bf16x8_t*)(q + (size_t)t * q_stride + (size_t)(kvh * G + r) * d + e);
     }
-    bf16x8_t kreg[2][NDT];
-    bf16x4_t vreg[2][NOT];
+    f32x4_t acc[NOT];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
+    for (int i = 0; i < NOT; ++i) acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    const int k_begin = ci * chunk;
+    const int k_end = min(k_begin + chunk, p + 1);
+    // Block ids come through the scalar cache (the index is made uniform for the compiler) and are asked
+    // for one step ahead: a vector load would queue behind the K and V loads in flight, and under load a
+    // load that the K and V loads depend on costs microseconds.
+    auto block_of = [&](int kt_any) -> int {
+      const int kt = __builtin_amdgcn_readfirstlane(kt_any);
+      return (kt <= p && kt + 15 >= lo && kt < k_end) ? table[kt / block_size] : 0;
+    };
+    int next_blk[2];
+    next_blk[0] = block_of(k_begin + wave * 32);
+    next_blk[1] = block_of(k_begin + wave * 32 + 16);
+    for (int k0 = k_begin + wave * 32; k0 < k_end; k0 += FD_WAVES * 32) {
+      const int blk_now[2] = {next_blk[0], next_blk[1]};
+      next_blk[0] = block_of(k0 + FD_WAVES * 32);
+      next_blk[1] = block_of(k0 + FD_WAVES * 32 + 16);
+      if (k0 + 31 < lo) continue;
+      // the two 16-key tiles of this step; a tile past the last key is not touched
+      bool live[2], edge[2];
+      const bf16_t* kb[2];
+      const bf16_t* vb[2];
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        kreg[tt][dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
-        if (live[tt] && dt * 32 + g * 8 < d) kreg[tt][dt] = *(const bf16x8_t*)(kb[tt] + dt * 512);
+      for (int tt = 0; tt < 2; ++tt) {
+        const int kt = k0 + tt * 16;
+        live[tt] = kt <= p && kt + 15 >= lo;
+        edge[tt] = kt + 15 > p || kt < lo;
+        const int blk = live[tt] ? blk_now[tt] : 0;
+        const size_t tile = ((size_t)blk * Hkv + kvh) * block_size * d + (size_t)((kt % block_size) >> 4) * 16 * d;
+        kb[tt] = kcache + tile + (g * 16 + r) * 8;        // chunk 4 dt + g of slot r
+        vb[tt] = vcache + tile + (g * 16 + r) * 4;        // slots 4g..4g+3 of row 16 ot + r
       }
+      bf16x8_t kreg[2][NDT];
+      bf16x4_t vreg[2][NOT];
 #pragma unroll
-      for (int ot = 0; ot < NOT; ++ot) {
-        vreg[tt][ot] = (bf16x4_t){0, 0, 0, 0};
-        if (live[tt] && ot * 16 < d) vreg[tt][ot] = *(const bf16x4_t*)(vb[tt] + ot * 256);
+      for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          kreg[tt][dt] = (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+          if (live[tt] && dt * 32 + g * 8 < d) kreg[tt][dt] = *(const bf16x8_t*)(kb[tt] + dt * 512);
+        }
+#pragma unroll
+        for (int ot = 0; ot < NOT; ++ot) {
+          vreg[tt][ot] = (bf16x4_t){0, 0, 0, 0};
+          if (live[tt] && ot * 16 < d) vreg[tt][ot] = *(const bf16x4_t*)(vb[tt] + ot * 256);
+        }
       }
-    }
-    f32x4_t s[2];
+      f32x4_t s[2];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      for (int tt = 0; tt < 2; ++tt) {
+        s[tt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-        if (dt * 32 < d) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[tt][dt], qreg[dt], s[tt], 0, 0, 0);
-    }
-    // mask and scale; keys outside [lo, p] get -inf, whatever bits their slots hold
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + tt * 16 + 4 * g + i;
-        const float v = (key <= p && key >= lo) ? s[tt][i] * scale_log2 : -INFINITY;
-        s[tt][i] = v;
-        tmax = fmaxf(tmax, v);
+        for (int dt = 0; dt < NDT; ++dt)
+          if (dt * 32 < d) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[tt][dt], qreg[dt], s[tt], 0, 0, 0);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
-    const float mn = fmaxf(m, tmax);              // finite: the step holds at least one visible key
-    const float corr = fd_exp2(m - mn);           // m = -inf gives 0
-    bf16x8_t pb;
-    float psum = 0.f;
+      // mask and scale; keys outside [lo, p] get -inf, whatever bits their slots hold
+      float tmax = -INFINITY;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float pr = fd_exp2(s[tt][i] - mn);  // masked: exp2(-inf) = 0
-        psum += pr;
-        pb[tt * 4 + i] = from_f32<bf16_t>(pr);
-      }
-    l = l * corr + psum;
-    m = mn;
-    // values of masked keys may be anything (a freed block's bits): zero them at the edges
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-      if (edge[tt]) {
+      for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + tt * 16 + 4 * g + i;
-          if (!(key <= p && key >= lo)) {
+          const float v = (key <= p && key >= lo) ? s[tt][i] * scale_log2 : -INFINITY;
+          s[tt][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
+      const float mn = fmaxf(m, tmax);              // finite: the step holds at least one visible key
+      const float corr = fd_exp2(m - mn);           // m = -inf gives 0
+      bf16x8_t pb;
+      float psum = 0.f;
 #pragma unroll
-            for (int ot = 0; ot < NOT; ++ot) vreg[tt][ot][i] = (bf16_t)0.f;
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pr = fd_exp2(s[tt][i] - mn);  // masked: exp2(-inf) = 0
+          psum += pr;
+          pb[tt * 4 + i] = from_f32<bf16_t>(pr);
+        }
+      l = l * corr + psum;
+      m = mn;
+      // values of masked keys may be anything (a freed block's bits): zero them at the edges
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+        if (edge[tt]) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = k0 + tt * 16 + 4 * g + i;
+            if (!(key <= p && key >= lo)) {
+#pragma unroll
+              for (int ot = 0; ot < NOT; ++ot) vreg[tt][ot][i] = (bf16_t)0.f;
+            }
           }
         }
-      }
 #pragma unroll
-    for (int ot = 0; ot < NOT; ++ot) {
-      if (ot * 16 < d) {
+      for (int ot = 0; ot < NOT; ++ot) {
+        if (ot * 16 < d) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[ot][i] *= corr;
-        const bf16x8_t a = {vreg[0][ot][0], vreg[0][ot][1], vreg[0][ot][2], vreg[0][ot][3],
-                            vreg[1][ot][0], vreg[1][ot][1], vreg[1][ot][2], vreg[1][ot][3]};
-        acc[ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[ot], 0, 0, 0);
+          for (int i = 0; i < 4; ++i) acc[ot][i] *= corr;
+          const bf16x8_t a = {vreg[0][ot][0], vreg[0][ot][1], vreg[0][ot][2], vreg[0][ot][3],
+                              vreg[1][ot][0], vreg[1][ot][1], vreg[1][ot][2], vreg[1][ot][3]};
+          acc[ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[ot], 0, 0, 0);
+        }
       }
     }
-  }
-  // lane groups hold partial sums of l over their own keys
-  l += __shfl_xor(l, 16, RA_WAVE);
-  l += __shfl_xor(l, 32, RA_WAVE);
+    // lane groups hold partial sums of l over their own keys
+    l += __shfl_xor(l, 16, RA_WAVE);
+    l += __shfl_xor(l, 32, RA_WAVE);
 
-  // merge the waves through LDS: lane (head r, group g) holds O^T rows 16 ot + 4 g + i
-  float* lds_o = lds;                                  // [waves][G][d]
-  float* lds_ml = lds + FD_WAVES * G * d;              // [waves][G][2]
-  if (r < G) {
+    // merge the waves through LDS: lane (head r, group g) holds O^T rows 16 ot + 4 g + i
+    float* lds_o = lds;                                  // [waves][G][d]
+    float* lds_ml = lds + FD_WAVES * G * d;              // [waves][G][2]
+    if (r < G) {
 #pragma unroll
-    for (int ot = 0; ot < NOT; ++ot)
-      if (ot * 16 < d) {
+      for (int ot = 0; ot < NOT; ++ot)
+        if (ot * 16 < d) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lds_o[((size_t)wave * G + r) * d + ot * 16 + 4 * g + i] = acc[ot][i];
-      }
-    if (g == 0) {
-      lds_ml[(wave * G + r) * 2] = m;
-      lds_ml[(wave * G + r) * 2 + 1] = l;
-    }
-  }
-  __syncthreads();
-  const size_t pair = (size_t)li * Hkv + kvh;
-  const size_t prow = (pair * max_chunks + (ci - c_first)) * G;      // [pair][chunk][head]
-  for (int idx = tid; idx < G * d; idx += FD_THREADS) {
-    const int h = idx / d, e = idx % d;
-    float mw = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < FD_WAVES; ++w) mw = fmaxf(mw, lds_ml[(w * G + h) * 2]);
-    float lt = 0.f, ot = 0.f;
-#pragma unroll
-    for (int w = 0; w < FD_WAVES; ++w) {
-      const float mwv = lds_ml[(w * G + h) * 2];
-      const float c = (mwv == -INFINITY) ? 0.f : fd_exp2(mwv - mw);
-      lt += lds_ml[(w * G + h) * 2 + 1] * c;
-      ot += lds_o[((size_t)w * G + h) * d + e] * c;
-    }
-    if (n_chunks == 1) {
-      out[(size_t)t * out_stride + (size_t)(kvh * G + h) * d + e] = from_f32<bf16_t>(ot / lt);
-    } else {
-      part_o[(prow + h) * d + e] = ot;
-      if (e == 0) {
-        part_ml[(prow + h) * 2] = mw;
-        part_ml[(prow + h) * 2 + 1] = lt;
+          for (int i = 0; i < 4; ++i) lds_o[((size_t)wave * G + r) * d + ot * 16 + 4 * g + i] = acc[ot][i];
+        }
+      if (g == 0) {
+        lds_ml[(wave * G + r) * 2] = m;
+        lds_ml[(wave * G + r) * 2 + 1] = l;
       }
     }
+    __syncthreads();
+    const size_t pair = (size_t)li * Hkv + kvh;
+    const size_t prow = (pair * max_chunks + (ci - c_first)) * G;      // [pair][chunk][head]
+    for (int idx = tid; idx < G * d; idx += FD_THREADS) {
+      const int h = idx / d, e = idx % d;
+      float mw = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < FD_WAVES; ++w) mw = fmaxf(mw, lds_ml[(w * G + h) * 2]);
+      float lt = 0.f, ot = 0.f;
+#pragma unroll
+      for (int w = 0; w < FD_WAVES; ++w) {
+        const float mwv = lds_ml[(w * G + h) * 2];
+        const float c = (mwv == -INFINITY) ? 0.f : fd_exp2(mwv - mw);
+        lt += lds_ml[(w * G + h) * 2 + 1] * c;
+        ot += lds_o[((size_t)w * G + h) * d + e] * c;
+      }
+      if (n_chunks == 1) {
+        out[(size_t)t * out_stride + (size_t)(kvh * G + h) * d + e] = from_f32<bf16_t>(ot / lt);
+      } else {
+        part_o[(prow + h) * d + e] = ot;
+        if (e == 0) {
+          part_ml[(prow + h) * 2] = mw;
+          part_ml[(prow + h) * 2 + 1] = lt;
+        }
+      }
+    }
+    __syncthreads();                                // the next item writes the same LDS
   }
 }
 
@@ -220,9 +277,9 @@ __global__ void __launch_bounds__(RA_WAVE)
 flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                           bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
                           const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk,
-                          int max_chunks) {
+                          int max_chunks, int t_base) {
   const int head = blockIdx.x, li = blockIdx.y;
-  const int t = token_list ? token_list[li] : li;
+  const int t = token_list ? token_list[li] : t_base + li;
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int n_chunks = p / chunk - lo / chunk + 1;
@@ -275,6 +332,25 @@ flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restr
   }
 }
 
+// Workgroups of the kernel that the current device holds at once (asked once a head-size variant and
+// LDS size; the answer of the first device stands for all: one kind of GPU in a process).
+static int fd_resident_workgroups(int variant, size_t lds) {
+  static int cached[3] = {0, 0, 0};
+  static size_t cached_lds[3] = {0, 0, 0};
+  if (cached[variant] > 0 && cached_lds[variant] == lds) return cached[variant];
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  hipError_t e = hipSuccess;
+  if (variant == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<64>, FD_THREADS, lds);
+  else if (variant == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<128>, FD_THREADS, lds);
+  else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<256>, FD_THREADS, lds);
+  if (e != hipSuccess || cus <= 0 || per_cu <= 0) return 0;
+  cached[variant] = cus * per_cu;
+  cached_lds[variant] = lds;
+  return cached[variant];
+}
+
 // 1 if the kernel takes these sizes, else 0 (the caller then uses the plain kernel)
 extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return 0;
@@ -301,27 +377,37 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   RA_CHECK(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                ((uintptr_t)vcache % 16) == 0,
            "attention_decode: operands must be 16-byte aligned");
-  RA_CHECK(n_tokens <= 65535 && Hkv <= 65535, "attention_decode: grid too large");
   const int G = Hq / Hkv;
-  dim3 grid(max_chunks, Hkv, n_tokens);
   const float scale_log2 = scale * 1.4426950408889634f;
   const size_t lds = (size_t)FD_WAVES * G * (d + 2) * sizeof(float);
   RA_CHECK(lds <= 64 * 1024, "attention_decode: %d heads of %d per KV head need too much LDS", G, d);
+  const int slots = fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, lds);
+  RA_CHECK(slots > 0, "attention_decode: cannot size the grid (%s)", hipGetErrorString(hipGetLastError()));
+  // lists longer than the kernel's item table go in slices, each with its part of the partial buffers
+  for (int base = 0; base < n_tokens; base += FD_MAX_TOKENS) {
+    const int n = n_tokens - base < FD_MAX_TOKENS ? n_tokens - base : FD_MAX_TOKENS;
+    const int* list = token_list ? token_list + base : nullptr;
+    const size_t rows = (size_t)base * Hkv * max_chunks * G;
+    float* po = part_o ? part_o + rows * d : nullptr;
+    float* pm = part_ml ? part_ml + rows * 2 : nullptr;
+    const long items_max = (long)n * Hkv * max_chunks;
+    const int grid = (int)(items_max < slots ? items_max : slots);
 #define RA_FD(DM)                                                                                     \
   flash_decode_kernel<DM><<<grid, FD_THREADS, lds, stream>>>(                                         \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
-      (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions,           \
-      block_size, Hkv, G, d, scale_log2, window, chunk, max_chunks, part_o, part_ml)
-  if (d <= 64) RA_FD(64);
-  else if (d <= 128) RA_FD(128);
-  else RA_FD(256);
+      (const bf16_t*)vcache, block_tables, max_blocks, list, seq_of_token, positions, block_size,     \
+      Hkv, G, d, scale_log2, window, chunk, max_chunks, n, base, po, pm)
+    if (d <= 64) RA_FD(64);
+    else if (d <= 128) RA_FD(128);
+    else RA_FD(256);
 #undef RA_FD
-  RA_LAUNCH_CHECK("attention_decode");
-  if (max_chunks > 1) {
-    dim3 mg(Hq, n_tokens);
-    flash_decode_merge_kernel<<<mg, RA_WAVE, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, token_list,
-                                                         positions, Hkv, G, d, window, chunk, max_chunks);
-    RA_LAUNCH_CHECK("attention_decode merge");
+    RA_LAUNCH_CHECK("attention_decode");
+    if (max_chunks > 1) {
+      dim3 mg(Hq, n);
+      flash_decode_merge_kernel<<<mg, RA_WAVE, 0, stream>>>(po, pm, (bf16_t*)out, out_stride, list, positions,
+                                                           Hkv, G, d, window, chunk, max_chunks, base);
+      RA_LAUNCH_CHECK("attention_decode merge");
+    }
   }
   return 0;
 }

@@ -250,9 +250,10 @@ class HipKernels:
 
     @staticmethod
     def decode_chunk(n_tokens: int, num_kv_heads: int, max_ctx: int):
-        """Keys per workgroup of the decode kernel, a multiple of 128: enough
-        workgroups to fill 256 CUs several times over. -> (chunk, chunks of max_ctx)"""
-        want = max(1, -(-2048 // max(1, n_tokens * num_kv_heads)))
+        """Keys per work item of the decode kernel, a multiple of 128: about two items for each
+        workgroup that the chip holds at once (its grid is that many workgroups, whatever the
+        batch). -> (chunk, chunks of max_ctx)"""
+        want = max(1, 1536 // max(1, n_tokens * num_kv_heads))
         chunk = -(-max_ctx // want)
         chunk = max(128, -(-chunk // 128) * 128)
         return chunk, max(1, -(-max_ctx // chunk))

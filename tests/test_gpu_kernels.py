@@ -530,6 +530,27 @@ def test_attention_decode(Hq, Hkv, d):
                 close(out, ref, 2 ** -7)     # probabilities and values are bfloat16 products summed in float
 
 
+def test_attention_decode_more_tokens_than_one_launch_numbers():
+    """The kernel numbers the work items of at most 1024 tokens a launch; longer
+    lists go in slices, with and without a token list."""
+    Hq, Hkv, d = 4, 2, 32
+    q_lens, starts = [700, 500], [5, 300]
+    q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=31)
+    batch = FakeBatch(q_lens, starts, tables)
+    T = sum(q_lens)
+    ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0)
+    out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().attention_decode(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0, chunk=128)
+    close(out, ref, 2 ** -7)
+    rows = list(range(T - 1, 60, -1))                      # 1139 tokens, in descending order
+    lst = torch.tensor(rows, dtype=torch.int32, device=DEV)
+    out = torch.full((T, Hq * d), 7.0, device=DEV, dtype=torch.bfloat16)
+    ops().attention_decode(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0, lst,
+                           len(rows), max(s + n for s, n in zip(starts, q_lens)), chunk=256)
+    close(out[rows], ref[rows], 2 ** -7)
+    assert (out[:61] == 7.0).all()
+
+
 def test_attention_decode_token_list_leaves_other_rows_alone():
     Hq, Hkv, d = 8, 2, 64
     q_lens, starts = [1, 6, 1], [40, 3, 99]
