@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 6
+#define RA_ABI_VERSION 7
 
 #ifdef __cplusplus
 extern "C" {
@@ -45,6 +45,16 @@ int ra_gemm_plain(const void* A, const void* W, const void* bias, void* C, int i
 int ra_gemm_skinny_max_rows(void);
 int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                    int M, int N, int K, int lda, int ldc, hipStream_t stream);
+// The same with an RMSNorm carried by the products around it, y = rstd[m] * ((x .* w) . W^T):
+// in_ss float [in_parts, M], if given: partial sums of squares of the rows behind A; the result
+// rows are scaled by rsqrt(sum / in_width + in_eps). out_w / out_x / out_ss, if given (epilogue 2
+// only): after C += ..., out_x[M, N] = bf16(C * out_w[n]) and out_ss[ra_gemm_skinny_row_parts(M, N), M]
+// = each workgroup's sums of squares of its columns of C.
+int ra_gemm_skinny_row_parts(int M, int N);
+int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                          int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
+                          int in_parts, float in_eps, int in_width, const void* out_w, int out_w_dtype,
+                          void* out_x, int out_ldx, float* out_ss, hipStream_t stream);
 
 // The cache of a layer: K and V are [blocks][Hkv][block_size * d], every (block, KV head) slab
 // in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);

@@ -339,16 +339,64 @@ class HipKernels:
                      _tag(x, "linear input"), _tag(out, "linear output"), M, N, K, x.stride(0),
                      out.stride(0), _stream())
 
-    def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False) -> None:
-        """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to."""
+    def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False, row_sums=None,
+                      emit=None) -> None:
+        """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to.
+
+        An RMSNorm can ride on the products around it, y = rstd[m] * ((x .* w) . W^T):
+        ``row_sums`` = (ss float32 [parts, M], eps, width) scales result row m by
+        rsqrt(sum_p ss[p, m] / width + eps); ``emit`` = (w [N], x_out bfloat16 [M, N],
+        ss_out float32 [skinny_row_parts(M, N), M]), with ``accumulate`` only, also writes
+        bf16(out * w) and each workgroup's sums of squares of its columns of ``out``."""
         M, N, K = self._check_linear(x, weight, out, bias)
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
         if accumulate and out.dtype != torch.float32:
             raise TypeError("linear_skinny: accumulation is into a float32 matrix")
-        library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
-                     _tag(out, "linear output"), 2 if accumulate else 0, M, N, K, x.stride(0), out.stride(0),
-                     _stream())
+        if row_sums is None and emit is None:
+            library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                         _tag(out, "linear output"), 2 if accumulate else 0, M, N, K, x.stride(0), out.stride(0),
+                         _stream())
+            return
+        self._skinny_normed(x, weight, bias, out, 2 if accumulate else 0, M, N, K, row_sums, emit)
+
+    # Rows up to which an RMSNorm rides on the products around it (``row_sums`` / ``emit``) rather
+    # than running as a kernel of its own. Measured on the Qwen3-8B shape: the decode step gains
+    # 4 % at 1 and 8 rows and 3 % at 16, and loses 3 % at 32 and 4 % at 64, where the products
+    # hold two and four row tiles in registers.
+    NORM_ON_PRODUCTS_ROWS = 16
+
+    def skinny_row_parts(self, M: int, N: int) -> int:
+        """Partial sums a row that ``linear_skinny(..., emit=)`` writes for an [M, N] result."""
+        return int(library.load().ra_gemm_skinny_row_parts(int(M), int(N)))
+
+    def _skinny_normed(self, x, weight, bias, out, epilogue, M, N, K, row_sums, emit) -> None:
+        ss = eps = width = None
+        parts = 0
+        if row_sums is not None:
+            ss, eps, width = row_sums
+            _dev(ss)
+            if ss.dtype != torch.float32 or ss.dim() != 2 or ss.shape[1] != M or not ss.is_contiguous():
+                raise ValueError(f"linear_skinny: row sums {tuple(ss.shape)} {ss.dtype}, expected float32 [parts, {M}]")
+            parts = ss.shape[0]
+        w = xo = so = None
+        if emit is not None:
+            if epilogue != 2:
+                raise ValueError("linear_skinny: only an accumulating product emits for a norm")
+            w, xo, so = emit
+            _dev(w, xo, so)
+            need = self.skinny_row_parts(M, N)
+            if w.shape != (N,) or not w.is_contiguous():
+                raise ValueError(f"linear_skinny: norm weight {tuple(w.shape)}, expected [{N}]")
+            if xo.dtype != torch.bfloat16 or xo.shape != (M, N) or xo.stride(1) != 1:
+                raise ValueError(f"linear_skinny: scaled copy {tuple(xo.shape)} {xo.dtype}, expected bfloat16 [{M}, {N}]")
+            if so.dtype != torch.float32 or so.shape != (need, M) or not so.is_contiguous():
+                raise ValueError(f"linear_skinny: emitted sums {tuple(so.shape)}, expected float32 [{need}, {M}]")
+        library.call("ra_gemm_skinny_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                     _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0),
+                     _ptr(ss), parts, float(eps or 0.0), int(width or 0), _ptr(w),
+                     _tag(w, "norm weight") if w is not None else 0, _ptr(xo),
+                     xo.stride(0) if xo is not None else 0, _ptr(so), _stream())
 
     def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
         """True if ``linear_skinny(..., accumulate=True)`` takes this product (out += x . W^T):
@@ -358,7 +406,7 @@ class HipKernels:
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 
-    def gated_linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+    def gated_linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, row_sums=None) -> None:
         """out[M, I] = silu(x . Wg^T) * (x . Wu^T) for ``weight`` [2I, K] whose rows alternate in
         runs of GATE_GROUP: 8 gate rows, the 8 up rows of the same features, and so on.
 
@@ -372,9 +420,14 @@ class HipKernels:
         if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 \
                 and M <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1 \
                 and weight.is_contiguous() and out.stride(1) == 1:
-            library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), None, out.data_ptr(),
-                         _tag(out, "linear output"), 1, M, 2 * I, K, x.stride(0), out.stride(0), _stream())
+            if row_sums is None:
+                library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), None, out.data_ptr(),
+                             _tag(out, "linear output"), 1, M, 2 * I, K, x.stride(0), out.stride(0), _stream())
+            else:
+                self._skinny_normed(x, weight, None, out, 1, M, 2 * I, K, row_sums, None)
             return
+        if row_sums is not None:
+            raise ValueError("gated_linear: row sums ride on the weight-streaming product only (bfloat16, <= 64 rows)")
         gu = torch.empty((M, 2 * I), dtype=out.dtype, device=x.device)
         self.linear(x, weight, gu)
         self.silu_mul(gu, out, self.GATE_GROUP)

@@ -59,8 +59,20 @@ class DecoderModel:
         resid = torch.empty((batch.num_tokens, self.spec.hidden), dtype=torch.float32, device=self.device)
         ops.embed(self.embed, batch.token_ids, resid)
         delta = None
+        n = len(self.run_order)
         for i, e in enumerate(self.run_order):
-            delta = self.blocks[e.block].forward(resid, delta, batch, caches[i])
+            block = self.blocks[e.block]
+            # the block that runs next may offer buffers that let this block's last product prepare
+            # its first norm
+            tgt = None
+            if i + 1 < n and getattr(block, "passes_emit", False):
+                nxt = self.blocks[self.run_order[i + 1].block]
+                if hasattr(nxt, "entry_target"):
+                    tgt = nxt.entry_target(resid)
+            if tgt is not None:
+                delta = block.forward(resid, delta, batch, caches[i], emit=tgt)
+            else:
+                delta = block.forward(resid, delta, batch, caches[i])
         return resid, delta
 
     def forward(self, batch, caches: Sequence[Optional[LayerCache]]) -> torch.Tensor:
@@ -69,6 +81,8 @@ class DecoderModel:
         The head runs on the wanted rows only (the reference computes all rows of
         a prompt and keeps the last, crates/cuda/src/engine.rs:5685-5720)."""
         resid, delta = self.forward_layers(batch, caches)
+        if delta is not None and not isinstance(delta, torch.Tensor):
+            delta = None               # a filled norm target: the sum is already in the stream
         xn = self.final_norm.add_norm(resid, delta, rows=batch.logit_rows)
         logits = torch.empty((batch.num_logit_rows, self.spec.vocab_size), dtype=torch.float32,
                              device=self.device)

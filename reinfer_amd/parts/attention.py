@@ -17,7 +17,7 @@ import torch
 from .. import kernels
 from ..config.schema import MixerSpec
 from ..weights import MATRIX, VECTOR, ParamDecl
-from .base import KVNeed, LayerCache
+from .base import KVNeed, LayerCache, NormTarget, split_input
 from .registry import lookup, register_mixer
 
 
@@ -25,6 +25,8 @@ from .registry import lookup, register_mixer
 class GroupedQueryAttention:
     graph_safe = True       # no host-side state: a decode step with it can be captured
     adds_in_place = True    # forward(..., resid=) may add the output projection into the stream
+    takes_row_scaled = True     # x may be RowScaled: the q/k/v product applies the row factor
+    emits_for_norm = True       # forward(..., emit=) may fill a NormTarget from the output projection
 
     @classmethod
     def declare_params(cls, spec: MixerSpec, prefix: str) -> List[ParamDecl]:
@@ -71,11 +73,16 @@ class GroupedQueryAttention:
     def cache_need(self) -> KVNeed:
         return KVNeed(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None):
+    def forward(self, x, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None,
+                emit: Optional[NormTarget] = None):
         ops = kernels.current()
+        x, row_sums = split_input(x)
         T = x.shape[0]
         qkv = torch.empty((T, self.qkv_width), dtype=self.dtype, device=x.device)
-        ops.linear(x, self.w_qkv, qkv, self.b_qkv)
+        if row_sums is None:
+            ops.linear(x, self.w_qkv, qkv, self.b_qkv)
+        else:
+            ops.linear_skinny(x, self.w_qkv, qkv, self.b_qkv, row_sums=row_sums)
         slots = batch.slots[cache.group] if cache.writes else batch.no_slots
         ops.qk_norm_rope_cache(qkv, self.q_norm, self.k_norm, self.eps, batch.positions,
                                self.position.inv_freq, self.position.rotary_dim, self.position.style,
@@ -85,7 +92,11 @@ class GroupedQueryAttention:
                       self.num_kv_heads, self.head_dim, self.scale, self.window, cache.group)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(attn, self.w_o):
-            ops.linear_skinny(attn, self.w_o, resid, accumulate=True)      # x += attn . Wo^T in the epilogue
+            # x += attn . Wo^T in the epilogue, which can also prepare the norm that follows
+            if emit is not None:
+                ops.linear_skinny(attn, self.w_o, resid, accumulate=True, emit=emit.emit)
+                return emit
+            ops.linear_skinny(attn, self.w_o, resid, accumulate=True)
             return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(attn, self.w_o, out)

@@ -41,16 +41,50 @@ class PreNormBlock:
                                                            p + spec.ffn_norm_name, dtype, device)
         self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
 
-    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch,
-                cache: Optional[LayerCache]) -> torch.Tensor:
+    passes_emit = True      # forward(..., emit=) hands a NormTarget on to the feed-forward
+
+    def entry_target(self, resid: torch.Tensor):
+        """A NormTarget for this block's first norm, for the part that runs before the block, or
+        None if the norm or the mixer behind it cannot use one."""
+        if not getattr(self.mixer, "takes_row_scaled", False) or not hasattr(self.mixer_norm, "emit_target"):
+            return None
+        return self.mixer_norm.emit_target(resid)
+
+    def forward(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache], emit=None):
         # A part that declares ``adds_in_place`` also gets the residual stream: where its last
         # product can add into it, it does and returns None; any other part returns its addend.
-        xn = self.mixer_norm.add_norm(resid, delta)
-        if getattr(self.mixer, "adds_in_place", False):
-            a = self.mixer.forward(xn, batch, cache, resid=resid)
+        # Where that product can also prepare the norm that follows (the part ``emits_for_norm``,
+        # the norm offers a target, and the part behind the norm ``takes_row_scaled``), the norm
+        # costs no kernel: its column weight is applied by the product before it, its row
+        # factor by the product after it.
+        mixer, ffn = self.mixer, self.ffn
+        xn = self._norm(self.mixer_norm, resid, delta, mixer)
+        if getattr(mixer, "adds_in_place", False):
+            tgt = self._target(self.ffn_norm, resid, mixer, ffn)
+            if tgt is not None:
+                a = mixer.forward(xn, batch, cache, resid=resid, emit=tgt)
+            else:
+                a = mixer.forward(xn, batch, cache, resid=resid)
         else:
-            a = self.mixer.forward(xn, batch, cache)
-        xn = self.ffn_norm.add_norm(resid, a)
-        if getattr(self.ffn, "adds_in_place", False):
-            return self.ffn.forward(xn, batch, resid=resid)
-        return self.ffn.forward(xn, batch)
+            a = mixer.forward(xn, batch, cache)
+        xn = self._norm(self.ffn_norm, resid, a, ffn)
+        if getattr(ffn, "adds_in_place", False):
+            if emit is not None and getattr(ffn, "emits_for_norm", False):
+                return ffn.forward(xn, batch, resid=resid, emit=emit)
+            return ffn.forward(xn, batch, resid=resid)
+        return ffn.forward(xn, batch)
+
+    @staticmethod
+    def _norm(norm, resid, delta, consumer):
+        if getattr(consumer, "takes_row_scaled", False) and hasattr(norm, "emit_target"):
+            return norm.add_norm(resid, delta, scaled_ok=True)
+        if not isinstance(delta, torch.Tensor) and delta is not None:
+            delta = None               # a filled target: the sum is already in the stream
+        return norm.add_norm(resid, delta)
+
+    @staticmethod
+    def _target(norm, resid, producer, consumer):
+        if not (getattr(producer, "emits_for_norm", False) and getattr(consumer, "takes_row_scaled", False)
+                and hasattr(norm, "emit_target")):
+            return None
+        return norm.emit_target(resid)

@@ -16,6 +16,7 @@ import torch
 from .. import kernels
 from ..config.schema import FeedForwardSpec
 from ..weights import ParamDecl
+from .base import NormTarget, split_input
 from .registry import register_feed_forward
 
 
@@ -23,6 +24,8 @@ from .registry import register_feed_forward
 class SwiGLU:
     graph_safe = True       # no host-side state: a decode step with it can be captured
     adds_in_place = True    # forward(..., resid=) may add the down projection into the stream
+    takes_row_scaled = True     # x may be RowScaled: the gate/up product applies the row factor
+    emits_for_norm = True       # forward(..., emit=) may fill a NormTarget from the down projection
 
     @classmethod
     def declare_params(cls, spec: FeedForwardSpec, prefix: str) -> List[ParamDecl]:
@@ -46,20 +49,31 @@ class SwiGLU:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = weights[prefix + "down_proj.weight"]
 
-    def forward(self, x: torch.Tensor, batch, resid: Optional[torch.Tensor] = None):
+    def forward(self, x, batch, resid: Optional[torch.Tensor] = None, emit: Optional[NormTarget] = None):
         ops = kernels.current()
+        x, row_sums = split_input(x)
         T = x.shape[0]
         I = self.spec.intermediate
         act = torch.empty((T, I), dtype=self.dtype, device=x.device)
         if self.group:
-            ops.gated_linear(x, self.w_gate_up, act)
+            if row_sums is None:
+                ops.gated_linear(x, self.w_gate_up, act)
+            else:
+                ops.gated_linear(x, self.w_gate_up, act, row_sums=row_sums)
         else:
             gu = torch.empty((T, 2 * I), dtype=self.dtype, device=x.device)
-            ops.linear(x, self.w_gate_up, gu)
+            if row_sums is None:
+                ops.linear(x, self.w_gate_up, gu)
+            else:
+                ops.linear_skinny(x, self.w_gate_up, gu, row_sums=row_sums)
             ops.silu_mul(gu, act)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(act, self.w_down):
-            ops.linear_skinny(act, self.w_down, resid, accumulate=True)    # x += act . Wd^T in the epilogue
+            # x += act . Wd^T in the epilogue, which can also prepare the norm that follows
+            if emit is not None:
+                ops.linear_skinny(act, self.w_down, resid, accumulate=True, emit=emit.emit)
+                return emit
+            ops.linear_skinny(act, self.w_down, resid, accumulate=True)
             return None
         out = torch.empty((T, self.spec.hidden), dtype=self.dtype, device=x.device)
         ops.linear(act, self.w_down, out)

@@ -12,6 +12,7 @@ import torch
 from .. import kernels
 from ..config.schema import NormSpec
 from ..weights import VECTOR, ParamDecl
+from .base import NormTarget, RowScaled
 from .registry import register_norm
 
 
@@ -28,14 +29,34 @@ class RMSNorm:
         self.weight = weights[name]
         self.dtype = dtype
 
-    def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
-                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def add_norm(self, resid: torch.Tensor, delta, rows: Optional[torch.Tensor] = None,
+                 scaled_ok: bool = False):
         """``resid += delta`` (float, in place) and the norm of the sum.
 
         With ``rows``, only those rows are computed, into a compact result, and
-        the residual is left as it is.
+        the residual is left as it is. ``delta`` may be None (nothing to add) or a
+        :class:`NormTarget` that the previous part filled for this norm: the sum is
+        in the stream already, and if the caller takes :class:`RowScaled`
+        (``scaled_ok``) there is nothing left to launch.
         """
+        if isinstance(delta, NormTarget):
+            if delta.norm is self and scaled_ok and rows is None:
+                return RowScaled(delta.x, delta.ss, self.eps, self.size)
+            delta = None
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=resid.device)
         kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
+
+    def emit_target(self, resid: torch.Tensor) -> Optional[NormTarget]:
+        """Buffers for a part that adds into ``resid`` with a product that can also prepare this
+        norm (bfloat16, few rows); None where that does not apply."""
+        ops = kernels.current()
+        parts = getattr(ops, "skinny_row_parts", None)
+        T = resid.shape[0]
+        if parts is None or self.dtype != torch.bfloat16 or T > getattr(ops, "NORM_ON_PRODUCTS_ROWS", 0) \
+                or resid.shape[1] != self.size:
+            return None
+        return NormTarget(self,
+                          torch.empty((T, self.size), dtype=torch.bfloat16, device=resid.device),
+                          torch.empty((parts(T, self.size), T), dtype=torch.float32, device=resid.device))

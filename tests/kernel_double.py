@@ -95,22 +95,46 @@ class KernelDouble:
             g, u = gate_up[:, :I].float(), gate_up[:, I:].float()
         out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
 
-    def gated_linear(self, x, weight, out):
-        gu = torch.empty((x.shape[0], weight.shape[0]), dtype=out.dtype)
+    def gated_linear(self, x, weight, out, row_sums=None):
+        gu = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32)
         self.linear(x, weight, gu)
-        self.silu_mul(gu, out, self.GATE_GROUP)
+        if row_sums is not None:
+            gu *= self._rstd(row_sums)[:, None]
+        self.silu_mul(gu.to(out.dtype), out, self.GATE_GROUP)
 
-    # the accumulating epilogue, so that the parts' use of it runs on the CPU too
+    # the accumulating epilogue and the norm that rides on products, so that the parts' use of
+    # them runs on the CPU too
     def can_accumulate(self, x, weight):
         return x.shape[0] <= 64
 
-    def linear_skinny(self, x, weight, out, bias=None, accumulate=False):
-        if not accumulate:
-            return self.linear(x, weight, out, bias)
+    ROW_PART = 16         # columns of one emitted partial sum
+    NORM_ON_PRODUCTS_ROWS = 64
+
+    def skinny_row_parts(self, M, N):
+        return -(-N // self.ROW_PART)
+
+    @staticmethod
+    def _rstd(row_sums):
+        ss, eps, width = row_sums
+        return torch.rsqrt(ss.double().sum(0) / width + eps).float()
+
+    def linear_skinny(self, x, weight, out, bias=None, accumulate=False, row_sums=None, emit=None):
         y = x.float() @ weight.float().T
+        if row_sums is not None:
+            y = y * self._rstd(row_sums)[:, None]
         if bias is not None:
             y = y + bias.float()
+        if not accumulate:
+            assert emit is None
+            out.copy_(y.to(out.dtype))
+            return
         out.add_(y.to(out.dtype))
+        if emit is not None:
+            w, xo, so = emit
+            xo.copy_((out.float() * w.float()).to(xo.dtype))
+            sq = out.float() ** 2
+            for p in range(so.shape[0]):
+                so[p] = sq[:, p * self.ROW_PART:(p + 1) * self.ROW_PART].sum(1)
 
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                   scale, window, group):

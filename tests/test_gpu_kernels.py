@@ -492,6 +492,47 @@ def test_gated_linear(M, I, K):
     close(out, g / (1 + torch.exp(-g)) * u, 2 ** -8 if M <= 64 else 3 * 2 ** -8)
 
 
+@pytest.mark.parametrize("M,N,K,wdt", [(1, 64, 64, torch.float32), (8, 4096, 1024, torch.float32),
+                                       (13, 200, 264, torch.bfloat16), (16, 96, 4096, torch.float32),
+                                       (23, 1000, 512, torch.bfloat16), (40, 328, 256, torch.float32),
+                                       (64, 9000, 128, torch.bfloat16), (64, 48, 1024, torch.float32)])
+def test_rmsnorm_carried_by_two_products(M, N, K, wdt):
+    """stream += a . W1^T, then y = rmsnorm(stream; w, eps) . W2^T with no norm kernel: the first
+    product also writes bf16(stream * w) and partial sums of squares, the second applies the
+    row factor; plain and gated second products, against the same in double precision."""
+    torch.manual_seed(M * 7 + N)
+    eps = 1e-5
+    a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    stream = torch.randn(M, N, device=DEV) * 3
+    stream[M // 2] *= 50                                       # one row far larger than the rest
+    nw = (1 + 0.3 * torch.randn(N, device=DEV)).to(wdt)
+    parts = ops().skinny_row_parts(M, N)
+    xs = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ss = torch.full((parts, M), float("nan"), device=DEV)
+    want_stream = stream.double() + a.double() @ w1.double().T
+    ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss))
+    close(stream, want_stream, 2 ** -8)
+    close(xs, stream.double() * nw.double(), 2 ** -8)
+    close(ss.sum(0), (stream.double() ** 2).sum(1), 1e-5)
+    normed = stream.double() * torch.rsqrt((stream.double() ** 2).mean(1, keepdim=True) + eps) * nw.double()
+    if N % 8 == 0:
+        J = 80
+        w2 = (torch.randn(J, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
+        bias = torch.randn(J, device=DEV).to(torch.bfloat16)
+        for dout in (torch.bfloat16, torch.float32):
+            y = torch.full((M, J), float("nan"), device=DEV, dtype=dout)
+            ops().linear_skinny(xs, w2, y, bias, row_sums=(ss, eps, N))
+            close(y, normed @ w2.double().T + bias.double(), 3 * 2 ** -8)
+        wg = (torch.randn(J, N, device=DEV) * 2 / math.sqrt(N)).to(torch.bfloat16)
+        wu = (torch.randn(J, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
+        w = torch.stack([wg.view(J // 8, 8, N), wu.view(J // 8, 8, N)], dim=1).reshape(2 * J, N).contiguous()
+        out = torch.full((M, J), float("nan"), device=DEV, dtype=torch.bfloat16)
+        ops().gated_linear(xs, w, out, row_sums=(ss, eps, N))
+        g, u = normed @ wg.double().T, normed @ wu.double().T
+        close(out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
+
+
 def test_linear_dispatch_refuses_nothing_silently():
     """Sizes the MFMA kernel does not take go to the plain kernel, not to a wrong result."""
     x = torch.randn(5, 100, device=DEV).to(torch.bfloat16)[:, :99]       # K = 99, odd row stride
