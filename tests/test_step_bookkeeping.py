@@ -127,3 +127,40 @@ def test_no_logits_wanted_still_stores(tmp_path):
         assert out.shape == (0, raw["vocab_size"])
         got = runner.step([StepEntry("a", toks[19:], [0])])
         assert rel_err(got, ref[19:]) < 2e-5
+
+
+class CountingDouble(KernelDouble):
+    def __init__(self, rows):
+        super().__init__()
+        self.NORM_ON_PRODUCTS_ROWS = rows
+        self.norm_calls = 0
+
+    def add_rmsnorm(self, *a, **k):
+        self.norm_calls += 1
+        return super().add_rmsnorm(*a, **k)
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_norm_carried_by_products_equals_norm_kernel(tmp_path, which):
+    """bfloat16, few rows: the parts hand the norm between layers to the products around it
+    (two norm launches a step remain: before the first layer and before the head). The logits
+    agree with the step that launches every norm, and with the plain implementation."""
+    folder = make_folder(tmp_path, which, "bfloat16")
+    raw, weights = read_folder(folder)
+    toks = random_tokens(23, raw["vocab_size"], 5)
+    ref = plain.forward(raw, weights, toks)
+    L = raw["num_hidden_layers"]
+    got = {}
+    for rows in (0, 64):
+        double = CountingDouble(rows)
+        with kernels.use(double):
+            runner = ModelRunner.from_folder(folder, dtype="bfloat16", device="cpu", max_tokens=128)
+            runner.add_request("a")
+            parts = [runner.step([StepEntry("a", toks[:9], list(range(9)))])]
+            for i in range(9, len(toks)):
+                parts.append(runner.step([StepEntry("a", toks[i:i + 1], [0])]))
+            got[rows] = torch.cat(parts)
+            steps = 1 + len(toks) - 9
+            assert double.norm_calls == steps * ((2 * L + 1) if rows == 0 else 2)
+    assert rel_err(got[64], got[0]) < 2e-2
+    assert rel_err(got[64], ref) < 3e-2 and rel_err(got[0], ref) < 3e-2
