@@ -1,0 +1,302 @@
+// Weight-streaming product for 17 to 64 rows:  C[M,N] = A[M,K] . W[N,K]^T, bfloat16 in, float
+// accumulation on the matrix cores.
+//
+// With more than one row tile the activations weigh as much as the weights: a workgroup that
+// owns 16 features and splits K over its waves (gemm_skinny.hip) reads all of A, once a wave
+// slice, and with its registers full of row tiles it keeps too few bytes in flight to cover the
+// memory latency (measured at 64 rows: 3 TB/s). Here the eight waves of a workgroup split the
+// features instead, 16 each, and walk K together: a run of 128 k of A is loaded once for the
+// whole workgroup into LDS (two buffers, one barrier a run), every wave streams its own 16
+// weight rows (contiguous 256-byte runs, re-laid through a tile of its own into MFMA layout),
+// and loads run three runs ahead of the matrix cores (more was measured: no faster).
+// A wave owns its 16 features over the
+// workgroup's whole K range, so there is nothing to add between waves.
+//
+// Where N gives too few workgroups of 128 features to fill the chip, K is cut into S ranges
+// (grid.y); each writes its float partial result and a second kernel adds them in range order
+// and applies the epilogue: deterministic, no atomics. Epilogues as in gemm_skinny.hip: plain
+// (+ bias), SiLU gate over interleaved gate/up rows (S = 1 only), C += (float).
+#include "common.h"
+#include "reinfer_hip.h"
+
+enum { WEPI_PLAIN = 0, WEPI_SILU_PAIRS = 1, WEPI_ACCUM = 2, WEPI_PARTIAL = 3 };
+
+#define GW_KS 128                      // k elements of a run
+#define GW_PITCH (GW_KS + 8)           // LDS row pitch in elements: 16 bytes of padding
+#ifndef GW_DEPTH
+#define GW_DEPTH 3                      // runs in flight ahead of the matrix cores
+#endif
+
+// WV waves a workgroup (8 or 6: 128 or 96 features; the host picks what fills the chip evenly)
+template <int MT, int WV>
+struct GwRegs {
+  bf16x8_t w[4];                                     // this wave's 16 weight rows x 128 k: 4 rows an instruction
+  bf16x8_t a[(MT * 16 + WV * 4 - 1) / (WV * 4)];     // the workgroup's MT*16 rows x 128 k: 4 WV rows a pass
+};
+
+template <int MT, int WV, int EPI, typename TO>
+__global__ void __launch_bounds__(WV * RA_WAVE)
+gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
+                 const bf16_t* __restrict__ bias, TO* __restrict__ C, int ldc, int M, int N, int K,
+                 int k_per_split) {
+  constexpr int RP = WV * 4;                     // rows of the A tile a pass of the whole workgroup loads
+  constexpr int AP = (MT * 16 + RP - 1) / RP;
+  constexpr int ATILE = MT * 16 * GW_PITCH;
+  constexpr int WTILE = 16 * GW_PITCH;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_a[2 * ATILE];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_w[WV * WTILE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
+  const int r = lane & 15, g = lane >> 4;        // MFMA operand layout
+  const int lr = lane >> 4, lc = lane & 15;      // weight loads: 16 lanes a row, 4 rows an instruction
+  const int ar = tid >> 4, ac = tid & 15;        // A loads: 16 threads a row, RP rows a pass
+  const int n0 = (blockIdx.x * WV + wave) * 16;
+  const int kb = blockIdx.y * k_per_split;
+  const int ke = min(K, kb + k_per_split);
+  const int n_runs = (ke - kb + GW_KS - 1) / GW_KS;
+  bf16_t* my_w = lds_w + wave * WTILE;
+
+  const bf16_t* wp[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int n = n0 + i * 4 + lr;
+    n = n < N ? n : N - 1;                       // rows past the end are computed and dropped
+    wp[i] = W + (size_t)n * K + kb + lc * 8;
+  }
+  const bf16_t* ap[AP];
+  bool aok[AP];
+#pragma unroll
+  for (int ps = 0; ps < AP; ++ps) {
+    int m = ps * RP + ar;
+    aok[ps] = m < M && m < MT * 16;              // rows past M are zeros, not loaded
+    m = m < M ? m : M - 1;
+    ap[ps] = A + (size_t)m * lda + kb + ac * 8;
+  }
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  auto gload = [&](GwRegs<MT, WV>& R, int run) {
+    const int k = run * GW_KS;
+    const bool wok = kb + k + lc * 8 < ke;       // K and the split are multiples of 8: a chunk is in or out
+    const bool kok = kb + k + ac * 8 < ke;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) R.w[i] = wok ? *(const bf16x8_t*)(wp[i] + k) : zero;
+#pragma unroll
+    for (int ps = 0; ps < AP; ++ps) R.a[ps] = (kok && aok[ps]) ? *(const bf16x8_t*)(ap[ps] + k) : zero;
+  };
+
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  // one run: registers -> LDS, ask for the run GW_DEPTH ahead into the same registers, barrier, multiply
+  auto step = [&](GwRegs<MT, WV>& R, int run) {
+    bf16_t* abuf = lds_a + (run & 1) * ATILE;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *(bf16x8_t*)(my_w + (i * 4 + lr) * GW_PITCH + lc * 8) = R.w[i];
+#pragma unroll
+    for (int ps = 0; ps < AP; ++ps)
+      if (ps * RP + ar < MT * 16) *(bf16x8_t*)(abuf + (ps * RP + ar) * GW_PITCH + ac * 8) = R.a[ps];
+    if (run + GW_DEPTH < n_runs) gload(R, run + GW_DEPTH);
+    // A buffer (run & 1) was last read in run - 2; every wave has passed the barrier of run - 1
+    // since, so it is free. This barrier makes the tile whole before anyone reads it.
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < GW_KS / 32; ++u) {
+      const bf16x8_t a = *(const bf16x8_t*)(my_w + r * GW_PITCH + u * 32 + g * 8);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8_t b = *(const bf16x8_t*)(abuf + (mt * 16 + r) * GW_PITCH + u * 32 + g * 8);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+      }
+    }
+    // the weight tile is the wave's own and is overwritten by the next run: its reads must be done
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+
+  GwRegs<MT, WV> R[GW_DEPTH];                       // indexed by constants only once unrolled: registers
+#pragma unroll
+  for (int d = 0; d < GW_DEPTH; ++d)
+    if (d < n_runs) gload(R[d], d);
+  for (int run = 0; run < n_runs; run += GW_DEPTH) {  // n_runs is the same in every thread of the workgroup
+#pragma unroll
+    for (int d = 0; d < GW_DEPTH; ++d)
+      if (run + d < n_runs) step(R[d], run + d);
+  }
+
+  // lane (r, g) holds C[feature n0 + 4g + i][token mt*16 + r]
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r;
+    if (EPI == WEPI_PARTIAL) {
+      if (m >= M) continue;
+      float* P = (float*)C + ((size_t)blockIdx.y * M + m) * N;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g + i;
+        if (n < N) P[n] = acc[mt][i];
+      }
+    } else if (EPI == WEPI_ACCUM || EPI == WEPI_PLAIN) {
+      if (m >= M) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g + i;
+        if (n >= N) continue;
+        float v = acc[mt][i];
+        if (bias) v += to_f32(bias[n]);
+        if (EPI == WEPI_ACCUM) v += to_f32(C[(size_t)m * ldc + n]);      // this thread alone owns (m, n)
+        C[(size_t)m * ldc + n] = from_f32<TO>(v);
+      }
+    } else {
+      // rows 0-7 of the wave's tile are gate, 8-15 up of the same features: the up value of
+      // gate row 4g + i sits in lane (r, g + 2), same i
+      float up[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) up[i] = __shfl_xor(acc[mt][i], 32, RA_WAVE);
+      if (m >= M || g >= 2) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int f = (n0 / 16) * 8 + 4 * g + i;
+        if (2 * f >= N) continue;              // N = 2 I
+        const float gt = acc[mt][i];
+        C[(size_t)m * ldc + f] = from_f32<TO>(gt / (1.f + __expf(-gt)) * up[i]);
+      }
+    }
+  }
+}
+
+// C = epilogue(sum over s of P[s]) for the K ranges of a split product, in range order.
+template <int EPI, typename TO>
+__global__ void __launch_bounds__(256)
+gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __restrict__ bias,
+                        TO* __restrict__ C, int ldc, int M, int N) {
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  const int m = blockIdx.y;
+  if (n >= N) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool whole = n + 3 < N && (N & 3) == 0;
+  for (int s = 0; s < S; ++s) {
+    const float* p = P + ((size_t)s * M + m) * N + n;
+    if (whole) {
+      const f32x4_t t = *(const f32x4_t*)p;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] += t[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) v[i] += p[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (n + i >= N) continue;
+    float x = v[i];
+    if (bias) x += to_f32(bias[n + i]);
+    if (EPI == WEPI_ACCUM) x += to_f32(C[(size_t)m * ldc + n + i]);
+    C[(size_t)m * ldc + n + i] = from_f32<TO>(x);
+  }
+}
+
+// How [M, N, K] is cut: waves a workgroup (8 or 6, 16 features each) and K ranges. With many features
+// one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
+// workgroups of 96). With few features 128 a workgroup and the smallest power of two up to 8 of K
+// ranges that gives at least 192 workgroups, each range a multiple of the run and two runs or more.
+static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_split) {
+  const int cb8 = (N + 127) / 128, cb6 = (N + 95) / 96;
+  *waves = 8;
+  *S = 1;
+  *k_per_split = (K + GW_KS - 1) / GW_KS * GW_KS;
+  if (cb8 >= 192 || epilogue == WEPI_SILU_PAIRS) {
+    const double e8 = (double)cb8 / (((cb8 + 255) / 256) * 256), e6 = (double)cb6 / (((cb6 + 255) / 256) * 256);
+    if (e6 > e8) *waves = 6;
+    return;
+  }
+  int s = 1;
+  while (s < 8 && cb8 * s < 192 && K / (s * 2) >= 2 * GW_KS) s *= 2;
+  int kps = (K + s - 1) / s;
+  kps = (kps + GW_KS - 1) / GW_KS * GW_KS;
+  *S = (K + kps - 1) / kps;
+  *k_per_split = kps;
+}
+
+// 1 where this kernel beats ra_gemm_skinny (measured on MI355X at 24 to 64 rows): from 17 rows on,
+// except a small product whose K has to be cut (4096 x 4096: the second launch costs more than the
+// shared activations save).
+extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
+  if (M < 17 || M > 64) return 0;
+  int waves, S, kps;
+  gw_split(epilogue, N, K, &waves, &S, &kps);
+  return (S == 1 || (long)N * K > 4096L * 4096L) ? 1 : 0;
+}
+
+// Floats of scratch that ra_gemm_wide needs for this product (0: none).
+extern "C" long ra_gemm_wide_scratch(int epilogue, int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int waves, S, kps;
+  gw_split(epilogue, N, K, &waves, &S, &kps);
+  return S > 1 ? (long)S * M * N : 0;
+}
+
+template <int MT, int WV>
+static int launch_wide(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int out_dtype,
+                       int epilogue, int M, int N, int K, int S, int kps, float* scratch, hipStream_t stream) {
+  const dim3 grid((N + WV * 16 - 1) / (WV * 16), S);
+#define RA_GW(EPI, TO, OUT, LD)                                                                 \
+  gemm_wide_kernel<MT, WV, EPI, TO><<<grid, WV * RA_WAVE, 0, stream>>>(                         \
+      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (TO*)(OUT), LD, M, N, K, kps)
+  if (S > 1) {
+    RA_GW(WEPI_PARTIAL, float, scratch, N);
+    RA_LAUNCH_CHECK("gemm_wide");
+    const dim3 rg((N + 1023) / 1024, M);
+#define RA_GR(EPI, TO) \
+  gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N)
+    if (epilogue == WEPI_ACCUM) RA_GR(WEPI_ACCUM, float);
+    else if (out_dtype == RA_BF16) RA_GR(WEPI_PLAIN, bf16_t);
+    else RA_GR(WEPI_PLAIN, float);
+#undef RA_GR
+    RA_LAUNCH_CHECK("gemm_wide reduce");
+    return 0;
+  }
+  if (epilogue == WEPI_SILU_PAIRS) {
+    if (out_dtype == RA_BF16) RA_GW(WEPI_SILU_PAIRS, bf16_t, C, ldc);
+    else RA_GW(WEPI_SILU_PAIRS, float, C, ldc);
+  } else if (epilogue == WEPI_ACCUM) {
+    RA_GW(WEPI_ACCUM, float, C, ldc);
+  } else {
+    if (out_dtype == RA_BF16) RA_GW(WEPI_PLAIN, bf16_t, C, ldc);
+    else RA_GW(WEPI_PLAIN, float, C, ldc);
+  }
+#undef RA_GW
+  RA_LAUNCH_CHECK("gemm_wide");
+  return 0;
+}
+
+extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
+                            int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
+                            hipStream_t stream) {
+  RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
+  RA_CHECK(M <= 64, "gemm_wide: %d rows; this kernel takes at most 64", M);
+  RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
+  RA_CHECK(epilogue == WEPI_PLAIN || epilogue == WEPI_SILU_PAIRS || epilogue == WEPI_ACCUM,
+           "gemm_wide: unknown epilogue %d", epilogue);
+  RA_CHECK(epilogue != WEPI_ACCUM || out_dtype == RA_F32, "gemm_wide: accumulation is into a float matrix");
+  const int n_out = epilogue == WEPI_SILU_PAIRS ? N / 2 : N;
+  RA_CHECK(epilogue != WEPI_SILU_PAIRS || (N % 16 == 0 && bias == nullptr),
+           "gemm_wide: the gated epilogue needs N (%d) in whole tiles of 16 and no bias", N);
+  RA_CHECK(lda >= K && ldc >= n_out, "gemm_wide: row strides (%d, %d) below the row lengths (%d, %d)", lda, ldc, K, n_out);
+  RA_CHECK(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_wide: operands must be 16-byte aligned");
+  RA_CHECK(out_dtype == RA_BF16 || out_dtype == RA_F32, "gemm_wide: unknown output dtype tag %d", out_dtype);
+  const long need = ra_gemm_wide_scratch(epilogue, M, N, K);
+  RA_CHECK(need == 0 || (scratch && scratch_floats >= need && ((uintptr_t)scratch % 16) == 0),
+           "gemm_wide: this product needs %ld floats of scratch, got %ld", need, scratch_floats);
+  int waves, S, kps;
+  gw_split(epilogue, N, K, &waves, &S, &kps);
+#define RA_GWL(MT)                                                                                            \
+  return waves == 6 ? launch_wide<MT, 6>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, stream) \
+                    : launch_wide<MT, 8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, stream)
+  if (M <= 16) RA_GWL(1);
+  if (M <= 32) RA_GWL(2);
+  if (M <= 48) RA_GWL(3);
+  RA_GWL(4);
+#undef RA_GWL
+}

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 7
+#define RA_ABI_VERSION 8
 
 #ifdef __cplusplus
 extern "C" {
@@ -55,6 +55,16 @@ int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* 
                           int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
                           int in_parts, float in_eps, int in_width, const void* out_w, int out_w_dtype,
                           void* out_x, int out_ldx, float* out_ss, hipStream_t stream);
+
+// bfloat16, up to 64 rows: the same product and epilogues with the activations shared by a
+// workgroup's waves; ra_gemm_wide_preferred says where it is the faster of the two (17 rows and
+// more, not the smallest products). Small N cuts K into ranges whose float partial results need
+// `ra_gemm_wide_scratch(...)` floats of scratch (0: none needed).
+int ra_gemm_wide_preferred(int epilogue, int M, int N, int K);
+long ra_gemm_wide_scratch(int epilogue, int M, int N, int K);
+int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
+                 int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
+                 hipStream_t stream);
 
 // The cache of a layer: K and V are [blocks][Hkv][block_size * d], every (block, KV head) slab
 // in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);

@@ -8,14 +8,14 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class KernelLibraryError(RuntimeError):
@@ -37,6 +37,7 @@ _SIGNATURES = {
     "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P, P],
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
+    "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
     "ra_gemm_skinny_normed": [P, P, P, P, I, I, I, I, I, I, I, P, I, F, I, P, I, P, I, P, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
@@ -73,6 +74,10 @@ def load() -> ctypes.CDLL:
         lib.ra_gemm_skinny_max_rows.argtypes = []
         lib.ra_gemm_skinny_row_parts.restype = c_int
         lib.ra_gemm_skinny_row_parts.argtypes = [c_int, c_int]
+        lib.ra_gemm_wide_scratch.restype = c_long
+        lib.ra_gemm_wide_scratch.argtypes = [c_int, c_int, c_int, c_int]
+        lib.ra_gemm_wide_preferred.restype = c_int
+        lib.ra_gemm_wide_preferred.argtypes = [c_int, c_int, c_int, c_int]
         if lib.ra_abi_version() != ABI_VERSION:
             raise KernelLibraryError(f"{path}: interface version {lib.ra_abi_version()}, expected {ABI_VERSION}; "
                                      "rebuild with `python -m reinfer_amd.csrc.build`")

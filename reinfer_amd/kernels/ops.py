@@ -340,7 +340,7 @@ class HipKernels:
                      out.stride(0), _stream())
 
     def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False, row_sums=None,
-                      emit=None) -> None:
+                      emit=None, wide: Optional[bool] = None) -> None:
         """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to.
 
         An RMSNorm can ride on the products around it, y = rstd[m] * ((x .* w) . W^T):
@@ -354,9 +354,7 @@ class HipKernels:
         if accumulate and out.dtype != torch.float32:
             raise TypeError("linear_skinny: accumulation is into a float32 matrix")
         if row_sums is None and emit is None:
-            library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
-                         _tag(out, "linear output"), 2 if accumulate else 0, M, N, K, x.stride(0), out.stride(0),
-                         _stream())
+            self._few_rows("linear output", x, weight, bias, out, 2 if accumulate else 0, M, N, K, wide)
             return
         self._skinny_normed(x, weight, bias, out, 2 if accumulate else 0, M, N, K, row_sums, emit)
 
@@ -365,6 +363,24 @@ class HipKernels:
     # 4 % at 1 and 8 rows and 3 % at 16, and loses 3 % at 32 and 4 % at 64, where the products
     # hold two and four row tiles in registers.
     NORM_ON_PRODUCTS_ROWS = 16
+
+    def _few_rows(self, what, x, weight, bias, out, epilogue, M, N, K, wide: Optional[bool] = None) -> None:
+        """The weight-streaming product for up to 64 rows, by one of two kernels: the one whose
+        waves split K (best up to 16 rows) or the one whose waves share the activations (it may
+        need scratch for partial sums). ``wide`` forces the choice; the library knows where each
+        is faster."""
+        lib = library.load()
+        if wide is None:
+            wide = bool(lib.ra_gemm_wide_preferred(epilogue, M, N, K))
+        if not wide:
+            library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                         _tag(out, what), epilogue, M, N, K, x.stride(0), out.stride(0), _stream())
+            return
+        need = int(lib.ra_gemm_wide_scratch(epilogue, M, N, K))
+        scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
+        library.call("ra_gemm_wide", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                     _tag(out, what), epilogue, M, N, K, x.stride(0), out.stride(0), _ptr(scratch), need,
+                     _stream())
 
     def skinny_row_parts(self, M: int, N: int) -> int:
         """Partial sums a row that ``linear_skinny(..., emit=)`` writes for an [M, N] result."""
@@ -406,7 +422,8 @@ class HipKernels:
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 
-    def gated_linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, row_sums=None) -> None:
+    def gated_linear(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, row_sums=None,
+                     wide: Optional[bool] = None) -> None:
         """out[M, I] = silu(x . Wg^T) * (x . Wu^T) for ``weight`` [2I, K] whose rows alternate in
         runs of GATE_GROUP: 8 gate rows, the 8 up rows of the same features, and so on.
 
@@ -421,8 +438,7 @@ class HipKernels:
                 and M <= 64 and K % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1 \
                 and weight.is_contiguous() and out.stride(1) == 1:
             if row_sums is None:
-                library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), None, out.data_ptr(),
-                             _tag(out, "linear output"), 1, M, 2 * I, K, x.stride(0), out.stride(0), _stream())
+                self._few_rows("linear output", x, weight, None, out, 1, M, 2 * I, K, wide)
             else:
                 self._skinny_normed(x, weight, None, out, 1, M, 2 * I, K, row_sums, None)
             return

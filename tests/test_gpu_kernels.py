@@ -448,35 +448,39 @@ def test_filtered_sampling_stays_inside_top_k():
 
 
 # ------------------------------------------------- bfloat16 kernels of serving
-@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 64])
-@pytest.mark.parametrize("N,K", [(100, 64), (333, 136), (1000, 96), (6144, 4096), (257, 520), (16, 8)])
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 40, 48, 49, 64])
+@pytest.mark.parametrize("N,K", [(100, 64), (333, 136), (1000, 96), (6144, 4096), (257, 520), (16, 8),
+                                 (48, 12288), (130, 1160)])
 @pytest.mark.parametrize("dout", ["bfloat16", "float32"])
-def test_linear_skinny(M, N, K, dout):
+@pytest.mark.parametrize("wide", [False, True])
+def test_linear_skinny(M, N, K, dout, wide):
+    """Both kernels for few rows (waves split K / waves share the activations), at every row count."""
     torch.manual_seed(M * N + K)
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
     b = torch.randn(N, device=DEV).to(torch.bfloat16)
     out = torch.full((M, N), float("nan"), device=DEV, dtype=DT[dout])
-    ops().linear_skinny(x, w, out)
+    ops().linear_skinny(x, w, out, wide=wide)
     ref = x.double() @ w.double().T
     close(out, ref, OUT_TOL[dout])
-    ops().linear_skinny(x, w, out, b)
+    ops().linear_skinny(x, w, out, b, wide=wide)
     close(out, ref + b.double(), OUT_TOL[dout])
     # the row of a token does not depend on its neighbours: row r of the batch = the single-row product
     one = torch.empty(1, N, device=DEV, dtype=DT[dout])
-    ops().linear_skinny(x[M - 1:M], w, one)
-    ops().linear_skinny(x, w, out)
+    ops().linear_skinny(x[M - 1:M], w, one, wide=wide)
+    ops().linear_skinny(x, w, out, wide=wide)
     close(one, out[M - 1:M], 1e-6 if dout == "float32" else 2 ** -8)
     # the accumulating epilogue: C += A . W^T into a float matrix
     c0 = torch.randn(M, N, device=DEV)
     c = c0.clone()
-    ops().linear_skinny(x, w, c, b, accumulate=True)
+    ops().linear_skinny(x, w, c, b, accumulate=True, wide=wide)
     close(c, c0.double() + ref + b.double(), 1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 20, 33, 64, 65, 200])
-@pytest.mark.parametrize("I,K", [(8, 8), (40, 64), (176, 80), (320, 96), (12288, 512)])
-def test_gated_linear(M, I, K):
+@pytest.mark.parametrize("M", [1, 7, 16, 20, 33, 48, 64, 65, 200])
+@pytest.mark.parametrize("I,K", [(8, 8), (40, 64), (176, 80), (320, 96), (12288, 512), (72, 1032)])
+@pytest.mark.parametrize("wide", [False, True])
+def test_gated_linear(M, I, K, wide):
     """silu(x Wg^T) * (x Wu^T) with gate and up rows interleaved in runs of 8: the fused epilogue
     (up to 64 rows) and the two-kernel form (more rows) against the separate float products."""
     torch.manual_seed(M + I + K)
@@ -485,7 +489,7 @@ def test_gated_linear(M, I, K):
     wu = (torch.randn(I, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
     w = torch.stack([wg.view(I // 8, 8, K), wu.view(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
     out = torch.full((M, I), float("nan"), device=DEV, dtype=torch.bfloat16)
-    ops().gated_linear(x, w, out)
+    ops().gated_linear(x, w, out, wide=wide if M <= 64 else None)
     g = x.double() @ wg.double().T
     u = x.double() @ wu.double().T
     # the two-kernel form rounds gate and up to bfloat16 before the gate: two more roundings
