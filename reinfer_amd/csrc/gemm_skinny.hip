@@ -351,6 +351,7 @@ extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* b
   }
   if (out_x || out_ss || out_w) {
     RA_CHECK(epilogue == EPI_ACCUM, "gemm_skinny: only the accumulating epilogue emits for a norm");
+    RA_CHECK(M <= 16, "gemm_skinny: with %d rows the other product kernel emits for a norm (this one up to 16)", M);
     RA_CHECK(out_x && out_ss && out_w, "gemm_skinny: emitting needs the norm weight, the scaled copy and the partial sums");
     RA_CHECK(out_w_dtype == RA_BF16 || out_w_dtype == RA_F32, "gemm_skinny: unknown norm weight dtype tag %d", out_w_dtype);
     RA_CHECK(out_ldx >= N, "gemm_skinny: the scaled copy's row stride (%d) is below %d", out_ldx, N);

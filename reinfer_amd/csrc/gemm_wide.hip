@@ -16,10 +16,33 @@
 // (grid.y); each writes its float partial result and a second kernel adds them in range order
 // and applies the epilogue: deterministic, no atomics. Epilogues as in gemm_skinny.hip: plain
 // (+ bias), SiLU gate over interleaved gate/up rows (S = 1 only), C += (float).
+//
+// An RMSNorm can ride on these products as on gemm_skinny's (y = rstd[m] * ((x .* w) . W^T)): the
+// row factor is applied in the epilogue of whichever kernel finishes the product; the scaled copy
+// and the partial sums of squares for the norm that follows an accumulating product are written by
+// the adding kernel, which such a product then always runs: one partial sum per row and 1024 columns.
 #include "common.h"
 #include "reinfer_hip.h"
 
 enum { WEPI_PLAIN = 0, WEPI_SILU_PAIRS = 1, WEPI_ACCUM = 2, WEPI_PARTIAL = 3 };
+
+// RMSNorm carried by the product (all pointers may be null): see gemm_skinny.hip
+struct WideNorm {
+  const float* in_ss;      // [in_parts, M] partial sums of squares of the rows behind A
+  int in_parts;
+  float in_eps, in_inv_width;
+  const void* out_w;       // [N] weight of the norm that follows (adding kernel only)
+  int out_w_f32;
+  bf16_t* out_x;           // [M, out_ldx] bf16(C_new * out_w)
+  int out_ldx;
+  float* out_ss;           // [ceil(N / 1024), M] sums of squares of C_new over 1024 columns
+};
+
+__device__ __forceinline__ float gw_rstd(const WideNorm& nf, int m, int M) {
+  float t = 0.f;
+  for (int p = 0; p < nf.in_parts; ++p) t += nf.in_ss[(size_t)p * M + m];      // fixed order
+  return rsqrtf(t * nf.in_inv_width + nf.in_eps);
+}
 
 #define GW_KS 128                      // k elements of a run
 #define GW_PITCH (GW_KS + 8)           // LDS row pitch in elements: 16 bytes of padding
@@ -38,7 +61,7 @@ template <int MT, int WV, int EPI, typename TO>
 __global__ void __launch_bounds__(WV * RA_WAVE)
 gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
                  const bf16_t* __restrict__ bias, TO* __restrict__ C, int ldc, int M, int N, int K,
-                 int k_per_split) {
+                 int k_per_split, WideNorm nf) {
   constexpr int RP = WV * 4;                     // rows of the A tile a pass of the whole workgroup loads
   constexpr int AP = (MT * 16 + RP - 1) / RP;
   constexpr int ATILE = MT * 16 * GW_PITCH;
@@ -128,6 +151,11 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
+    if (EPI != WEPI_PARTIAL && nf.in_ss && m < M) {      // a split product is scaled when its parts are added
+      const float rstd = gw_rstd(nf, m, M);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[mt][i] *= rstd;
+    }
     if (EPI == WEPI_PARTIAL) {
       if (m >= M) continue;
       float* P = (float*)C + ((size_t)blockIdx.y * M + m) * N;
@@ -165,35 +193,50 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   }
 }
 
-// C = epilogue(sum over s of P[s]) for the K ranges of a split product, in range order.
+// C = epilogue(sum over s of P[s]) for the K ranges of a split product, in range order; a workgroup
+// takes 1024 columns of one row. The carried norm's row factor and, for the norm that follows an
+// accumulating product, the scaled copy and the workgroup's sum of squares are applied here.
 template <int EPI, typename TO>
 __global__ void __launch_bounds__(256)
 gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __restrict__ bias,
-                        TO* __restrict__ C, int ldc, int M, int N) {
+                        TO* __restrict__ C, int ldc, int M, int N, WideNorm nf) {
+  __shared__ float red[17];
   const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   const int m = blockIdx.y;
-  if (n >= N) return;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
-  const bool whole = n + 3 < N && (N & 3) == 0;
-  for (int s = 0; s < S; ++s) {
-    const float* p = P + ((size_t)s * M + m) * N + n;
-    if (whole) {
-      const f32x4_t t = *(const f32x4_t*)p;
+  if (n < N) {
+    const bool whole = n + 3 < N && (N & 3) == 0;
+    for (int s = 0; s < S; ++s) {
+      const float* p = P + ((size_t)s * M + m) * N + n;
+      if (whole) {
+        const f32x4_t t = *(const f32x4_t*)p;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] += t[i];
-    } else {
+        for (int i = 0; i < 4; ++i) v[i] += t[i];
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < N) v[i] += p[i];
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) v[i] += p[i];
+      }
     }
   }
+  const float rstd = nf.in_ss ? gw_rstd(nf, m, M) : 1.f;
+  float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     if (n + i >= N) continue;
-    float x = v[i];
+    float x = v[i] * rstd;
     if (bias) x += to_f32(bias[n + i]);
     if (EPI == WEPI_ACCUM) x += to_f32(C[(size_t)m * ldc + n + i]);
     C[(size_t)m * ldc + n + i] = from_f32<TO>(x);
+    if (EPI == WEPI_ACCUM && nf.out_x) {
+      const float w = nf.out_w_f32 ? ((const float*)nf.out_w)[n + i] : to_f32(((const bf16_t*)nf.out_w)[n + i]);
+      nf.out_x[(size_t)m * nf.out_ldx + n + i] = from_f32<bf16_t>(x * w);
+      ss += x * x;
+    }
+  }
+  if (EPI == WEPI_ACCUM && nf.out_x) {        // the same for every thread of the workgroup
+    ss = block_sum(ss, red);
+    if (threadIdx.x == 0) nf.out_ss[(size_t)blockIdx.x * M + m] = ss;
   }
 }
 
@@ -201,12 +244,14 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
 // one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
 // workgroups of 96). With few features 128 a workgroup and the smallest power of two up to 8 of K
 // ranges that gives at least 192 workgroups, each range a multiple of the run and two runs or more.
-static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_split) {
+static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_split, bool* partial = nullptr,
+                     bool emits = false) {
+  if (partial) *partial = emits;                       // the adding kernel writes what the next norm needs
   const int cb8 = (N + 127) / 128, cb6 = (N + 95) / 96;
   *waves = 8;
   *S = 1;
   *k_per_split = (K + GW_KS - 1) / GW_KS * GW_KS;
-  if (cb8 >= 192 || epilogue == WEPI_SILU_PAIRS) {
+  if ((cb8 >= 192 && !emits) || epilogue == WEPI_SILU_PAIRS) {
     const double e8 = (double)cb8 / (((cb8 + 255) / 256) * 256), e6 = (double)cb6 / (((cb6 + 255) / 256) * 256);
     if (e6 > e8) *waves = 6;
     return;
@@ -217,6 +262,7 @@ static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_
   kps = (kps + GW_KS - 1) / GW_KS * GW_KS;
   *S = (K + kps - 1) / kps;
   *k_per_split = kps;
+  if (partial) *partial = emits || *S > 1;
 }
 
 // 1 where this kernel beats ra_gemm_skinny (measured on MI355X at 24 to 64 rows): from 17 rows on,
@@ -230,26 +276,31 @@ extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
 }
 
 // Floats of scratch that ra_gemm_wide needs for this product (0: none).
-extern "C" long ra_gemm_wide_scratch(int epilogue, int M, int N, int K) {
+extern "C" long ra_gemm_wide_scratch(int epilogue, int M, int N, int K, int emits) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   int waves, S, kps;
-  gw_split(epilogue, N, K, &waves, &S, &kps);
-  return S > 1 ? (long)S * M * N : 0;
+  bool partial;
+  gw_split(epilogue, N, K, &waves, &S, &kps, &partial, emits != 0);
+  return partial ? (long)S * M * N : 0;
 }
+
+// Partial sums a row that an emitting product writes for the norm that follows an [M, N] result.
+extern "C" int ra_gemm_wide_row_parts(int N) { return (N + 1023) / 1024; }
 
 template <int MT, int WV>
 static int launch_wide(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int out_dtype,
-                       int epilogue, int M, int N, int K, int S, int kps, float* scratch, hipStream_t stream) {
+                       int epilogue, int M, int N, int K, int S, int kps, bool partial, float* scratch,
+                       const WideNorm& nf, hipStream_t stream) {
   const dim3 grid((N + WV * 16 - 1) / (WV * 16), S);
 #define RA_GW(EPI, TO, OUT, LD)                                                                 \
   gemm_wide_kernel<MT, WV, EPI, TO><<<grid, WV * RA_WAVE, 0, stream>>>(                         \
-      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (TO*)(OUT), LD, M, N, K, kps)
-  if (S > 1) {
+      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (TO*)(OUT), LD, M, N, K, kps, nf)
+  if (partial) {
     RA_GW(WEPI_PARTIAL, float, scratch, N);
     RA_LAUNCH_CHECK("gemm_wide");
     const dim3 rg((N + 1023) / 1024, M);
 #define RA_GR(EPI, TO) \
-  gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N)
+  gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N, nf)
     if (epilogue == WEPI_ACCUM) RA_GR(WEPI_ACCUM, float);
     else if (out_dtype == RA_BF16) RA_GR(WEPI_PLAIN, bf16_t);
     else RA_GR(WEPI_PLAIN, float);
@@ -271,9 +322,11 @@ static int launch_wide(const void* A, int lda, const void* W, const void* bias, 
   return 0;
 }
 
-extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
-                            int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
-                            hipStream_t stream) {
+extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
+                                   int epilogue, int M, int N, int K, int lda, int ldc, float* scratch,
+                                   long scratch_floats, const float* in_ss, int in_parts, float in_eps,
+                                   int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
+                                   float* out_ss, hipStream_t stream) {
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
   RA_CHECK(M <= 64, "gemm_wide: %d rows; this kernel takes at most 64", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
@@ -286,17 +339,45 @@ extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void
   RA_CHECK(lda >= K && ldc >= n_out, "gemm_wide: row strides (%d, %d) below the row lengths (%d, %d)", lda, ldc, K, n_out);
   RA_CHECK(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_wide: operands must be 16-byte aligned");
   RA_CHECK(out_dtype == RA_BF16 || out_dtype == RA_F32, "gemm_wide: unknown output dtype tag %d", out_dtype);
-  const long need = ra_gemm_wide_scratch(epilogue, M, N, K);
+  WideNorm nf = {};
+  if (in_ss) {
+    RA_CHECK(in_parts > 0 && in_width > 0 && in_eps >= 0.f, "gemm_wide: row sums need parts (%d), width (%d) and eps", in_parts, in_width);
+    nf.in_ss = in_ss;
+    nf.in_parts = in_parts;
+    nf.in_eps = in_eps;
+    nf.in_inv_width = 1.f / (float)in_width;
+  }
+  const bool emits = out_x || out_ss || out_w;
+  if (emits) {
+    RA_CHECK(epilogue == WEPI_ACCUM, "gemm_wide: only the accumulating epilogue emits for a norm");
+    RA_CHECK(out_x && out_ss && out_w, "gemm_wide: emitting needs the norm weight, the scaled copy and the partial sums");
+    RA_CHECK(out_w_dtype == RA_BF16 || out_w_dtype == RA_F32, "gemm_wide: unknown norm weight dtype tag %d", out_w_dtype);
+    RA_CHECK(out_ldx >= N, "gemm_wide: the scaled copy's row stride (%d) is below %d", out_ldx, N);
+    nf.out_w = out_w;
+    nf.out_w_f32 = out_w_dtype == RA_F32;
+    nf.out_x = (bf16_t*)out_x;
+    nf.out_ldx = out_ldx;
+    nf.out_ss = out_ss;
+  }
+  const long need = ra_gemm_wide_scratch(epilogue, M, N, K, emits);
   RA_CHECK(need == 0 || (scratch && scratch_floats >= need && ((uintptr_t)scratch % 16) == 0),
            "gemm_wide: this product needs %ld floats of scratch, got %ld", need, scratch_floats);
   int waves, S, kps;
-  gw_split(epilogue, N, K, &waves, &S, &kps);
+  bool partial;
+  gw_split(epilogue, N, K, &waves, &S, &kps, &partial, emits);
 #define RA_GWL(MT)                                                                                            \
-  return waves == 6 ? launch_wide<MT, 6>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, stream) \
-                    : launch_wide<MT, 8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, stream)
+  return waves == 6 ? launch_wide<MT, 6>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream) \
+                    : launch_wide<MT, 8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream)
   if (M <= 16) RA_GWL(1);
   if (M <= 32) RA_GWL(2);
   if (M <= 48) RA_GWL(3);
   RA_GWL(4);
 #undef RA_GWL
+}
+
+extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
+                            int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
+                            hipStream_t stream) {
+  return ra_gemm_wide_normed(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, scratch, scratch_floats,
+                             nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, stream);
 }

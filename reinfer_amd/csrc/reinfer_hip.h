@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 8
+#define RA_ABI_VERSION 9
 
 #ifdef __cplusplus
 extern "C" {
@@ -48,8 +48,8 @@ int ra_gemm_skinny(const void* A, const void* W, const void* bias, void* C, int 
 // The same with an RMSNorm carried by the products around it, y = rstd[m] * ((x .* w) . W^T):
 // in_ss float [in_parts, M], if given: partial sums of squares of the rows behind A; the result
 // rows are scaled by rsqrt(sum / in_width + in_eps). out_w / out_x / out_ss, if given (epilogue 2
-// only): after C += ..., out_x[M, N] = bf16(C * out_w[n]) and out_ss[ra_gemm_skinny_row_parts(M, N), M]
-// = each workgroup's sums of squares of its columns of C.
+// only, up to 16 rows): after C += ..., out_x[M, N] = bf16(C * out_w[n]) and
+// out_ss[ra_gemm_skinny_row_parts(M, N), M] = each workgroup's sums of squares of its columns of C.
 int ra_gemm_skinny_row_parts(int M, int N);
 int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype,
                           int epilogue, int M, int N, int K, int lda, int ldc, const float* in_ss,
@@ -61,10 +61,17 @@ int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* 
 // more, not the smallest products). Small N cuts K into ranges whose float partial results need
 // `ra_gemm_wide_scratch(...)` floats of scratch (0: none needed).
 int ra_gemm_wide_preferred(int epilogue, int M, int N, int K);
-long ra_gemm_wide_scratch(int epilogue, int M, int N, int K);
+long ra_gemm_wide_scratch(int epilogue, int M, int N, int K, int emits);
 int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                  int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                  hipStream_t stream);
+// With a carried RMSNorm, as ra_gemm_skinny_normed; an emitting product always needs scratch
+// (ra_gemm_wide_scratch with emits = 1) and writes out_ss[ra_gemm_wide_row_parts(N), M].
+int ra_gemm_wide_row_parts(int N);
+int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
+                        int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
+                        const float* in_ss, int in_parts, float in_eps, int in_width, const void* out_w,
+                        int out_w_dtype, void* out_x, int out_ldx, float* out_ss, hipStream_t stream);
 
 // The cache of a layer: K and V are [blocks][Hkv][block_size * d], every (block, KV head) slab
 // in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 class KernelLibraryError(RuntimeError):
@@ -38,6 +38,7 @@ _SIGNATURES = {
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
+    "ra_gemm_wide_normed": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P, I, F, I, P, I, P, I, P, P],
     "ra_gemm_skinny_normed": [P, P, P, P, I, I, I, I, I, I, I, P, I, F, I, P, I, P, I, P, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
@@ -75,7 +76,9 @@ def load() -> ctypes.CDLL:
         lib.ra_gemm_skinny_row_parts.restype = c_int
         lib.ra_gemm_skinny_row_parts.argtypes = [c_int, c_int]
         lib.ra_gemm_wide_scratch.restype = c_long
-        lib.ra_gemm_wide_scratch.argtypes = [c_int, c_int, c_int, c_int]
+        lib.ra_gemm_wide_scratch.argtypes = [c_int, c_int, c_int, c_int, c_int]
+        lib.ra_gemm_wide_row_parts.restype = c_int
+        lib.ra_gemm_wide_row_parts.argtypes = [c_int]
         lib.ra_gemm_wide_preferred.restype = c_int
         lib.ra_gemm_wide_preferred.argtypes = [c_int, c_int, c_int, c_int]
         if lib.ra_abi_version() != ABI_VERSION:

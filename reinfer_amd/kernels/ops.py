@@ -359,10 +359,11 @@ class HipKernels:
         self._skinny_normed(x, weight, bias, out, 2 if accumulate else 0, M, N, K, row_sums, emit)
 
     # Rows up to which an RMSNorm rides on the products around it (``row_sums`` / ``emit``) rather
-    # than running as a kernel of its own. Measured on the Qwen3-8B shape: the decode step gains
-    # 4 % at 1 and 8 rows and 3 % at 16, and loses 3 % at 32 and 4 % at 64, where the products
-    # hold two and four row tiles in registers.
-    NORM_ON_PRODUCTS_ROWS = 16
+    # than running as a kernel of its own: all that the weight-streaming products take. Up to 16
+    # rows the kernel whose waves split K carries it, above that the other one, which has the
+    # registers to spare (the first, at 32 and 64 rows, got slower than with a norm kernel).
+    NORM_ON_PRODUCTS_ROWS = 64
+    NORM_SKINNY_ROWS = 16
 
     def _few_rows(self, what, x, weight, bias, out, epilogue, M, N, K, wide: Optional[bool] = None) -> None:
         """The weight-streaming product for up to 64 rows, by one of two kernels: the one whose
@@ -376,7 +377,7 @@ class HipKernels:
             library.call("ra_gemm_skinny", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                          _tag(out, what), epilogue, M, N, K, x.stride(0), out.stride(0), _stream())
             return
-        need = int(lib.ra_gemm_wide_scratch(epilogue, M, N, K))
+        need = int(lib.ra_gemm_wide_scratch(epilogue, M, N, K, 0))
         scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
         library.call("ra_gemm_wide", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                      _tag(out, what), epilogue, M, N, K, x.stride(0), out.stride(0), _ptr(scratch), need,
@@ -384,7 +385,10 @@ class HipKernels:
 
     def skinny_row_parts(self, M: int, N: int) -> int:
         """Partial sums a row that ``linear_skinny(..., emit=)`` writes for an [M, N] result."""
-        return int(library.load().ra_gemm_skinny_row_parts(int(M), int(N)))
+        lib = library.load()
+        if M <= self.NORM_SKINNY_ROWS:
+            return int(lib.ra_gemm_skinny_row_parts(int(M), int(N)))
+        return int(lib.ra_gemm_wide_row_parts(int(N)))
 
     def _skinny_normed(self, x, weight, bias, out, epilogue, M, N, K, row_sums, emit) -> None:
         ss = eps = width = None
@@ -408,11 +412,19 @@ class HipKernels:
                 raise ValueError(f"linear_skinny: scaled copy {tuple(xo.shape)} {xo.dtype}, expected bfloat16 [{M}, {N}]")
             if so.dtype != torch.float32 or so.shape != (need, M) or not so.is_contiguous():
                 raise ValueError(f"linear_skinny: emitted sums {tuple(so.shape)}, expected float32 [{need}, {M}]")
-        library.call("ra_gemm_skinny_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
-                     _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0),
-                     _ptr(ss), parts, float(eps or 0.0), int(width or 0), _ptr(w),
+        norm_args = (_ptr(ss), parts, float(eps or 0.0), int(width or 0), _ptr(w),
                      _tag(w, "norm weight") if w is not None else 0, _ptr(xo),
-                     xo.stride(0) if xo is not None else 0, _ptr(so), _stream())
+                     xo.stride(0) if xo is not None else 0, _ptr(so))
+        if M <= self.NORM_SKINNY_ROWS:
+            library.call("ra_gemm_skinny_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                         _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), *norm_args,
+                         _stream())
+            return
+        need = int(library.load().ra_gemm_wide_scratch(epilogue, M, N, K, 1 if emit is not None else 0))
+        scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
+        library.call("ra_gemm_wide_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                     _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), _ptr(scratch),
+                     need, *norm_args, _stream())
 
     def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
         """True if ``linear_skinny(..., accumulate=True)`` takes this product (out += x . W^T):

@@ -111,7 +111,10 @@ class KernelDouble:
     NORM_ON_PRODUCTS_ROWS = 64
 
     def skinny_row_parts(self, M, N):
-        return -(-N // self.ROW_PART)
+        return -(-N // self._row_part(M))
+
+    def _row_part(self, M):
+        return self.ROW_PART if M <= 16 else 1024
 
     @staticmethod
     def _rstd(row_sums):
@@ -133,8 +136,9 @@ class KernelDouble:
             w, xo, so = emit
             xo.copy_((out.float() * w.float()).to(xo.dtype))
             sq = out.float() ** 2
+            part = self._row_part(x.shape[0])
             for p in range(so.shape[0]):
-                so[p] = sq[:, p * self.ROW_PART:(p + 1) * self.ROW_PART].sum(1)
+                so[p] = sq[:, p * part:(p + 1) * part].sum(1)
 
     def attention(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                   scale, window, group):
