@@ -172,6 +172,35 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     for (int kp = 0; kp < 2; ++kp) {
       const int kh = k0 + kp * 32;
       if (kh > w_last_pos) break;          // the second half may lie past the wave's last query
+      // All LDS operands of the half are asked for at once, before the first matrix product: K for
+      // the scores and V for the output, which does not depend on the softmax in between (left to
+      // itself the compiler reads one operand, waits for it, multiplies, and so on: sixteen exposed
+      // LDS latencies a half; asking first made the kernel 12 % faster). Head sizes above 128 have
+      // no registers for that and read as they go.
+      constexpr bool AHEAD = DMAX <= 128;
+      const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+      auto k_operand = [&](int ks, int dt) -> bf16x8_t {
+        const int e = dt * 32 + g * 8;
+        return (e < d) ? *(const bf16x8_t*)(Ks + (kp * 2 + ks) * 16 * d + ((dt * 4 + g) * 16 + r) * 8) : zero8;
+      };
+      auto v_operand = [&](int ot, int hi) -> bf16x4_t {
+        const bf16_t* v0 = Vs + (2 * kp + hi) * 16 * d + ((ot * 4 + g) * 16 + r) * 4;
+        return (ot * 16 < d) ? *(const bf16x4_t*)(v0) : (bf16x4_t){0, 0, 0, 0};
+      };
+      bf16x8_t ka[AHEAD ? 2 : 1][AHEAD ? NDT : 1];
+      bf16x4_t vlo[AHEAD ? NOT : 1], vhi[AHEAD ? NOT : 1];
+      if constexpr (AHEAD) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int dt = 0; dt < NDT; ++dt) ka[ks][dt] = k_operand(ks, dt);
+#pragma unroll
+        for (int ot = 0; ot < NOT; ++ot) {
+          vlo[ot] = v_operand(ot, 0);
+          vhi[ot] = v_operand(ot, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);     // the reads stay ahead of the products
+      }
       // scores S^T[key][column] for 2 sub-tiles of 16 keys
       f32x4_t s[2][NC];
 #pragma unroll
@@ -181,9 +210,9 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
           if (dt * 32 < d) {
-            const int e = dt * 32 + g * 8;
-            const bf16x8_t a = (e < d) ? *(const bf16x8_t*)(Ks + (kp * 2 + ks) * 16 * d + ((dt * 4 + g) * 16 + r) * 8)
-                                       : (bf16x8_t){0, 0, 0, 0, 0, 0, 0, 0};
+            bf16x8_t a;
+            if constexpr (AHEAD) a = ka[ks][dt];
+            else a = k_operand(ks, dt);
 #pragma unroll
             for (int j = 0; j < NC; ++j)
               s[ks][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j][dt], s[ks][j], 0, 0, 0);
@@ -245,9 +274,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
       for (int ot = 0; ot < NOT; ++ot) {
         if (ot * 16 < d) {
-          const bf16_t* v0 = Vs + (2 * kp) * 16 * d + ((ot * 4 + g) * 16 + r) * 4;
-          const bf16x4_t lo4 = *(const bf16x4_t*)(v0);
-          const bf16x4_t hi4 = *(const bf16x4_t*)(v0 + 16 * d);
+          bf16x4_t lo4, hi4;
+          if constexpr (AHEAD) {
+            lo4 = vlo[ot];
+            hi4 = vhi[ot];
+          } else {
+            lo4 = v_operand(ot, 0);
+            hi4 = v_operand(ot, 1);
+          }
           const bf16x8_t a = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
 #pragma unroll
           for (int j = 0; j < NC; ++j)
