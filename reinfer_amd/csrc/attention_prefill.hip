@@ -10,8 +10,9 @@
 // (they were stored before this kernel runs), 64 keys a round, copied to LDS
 // as the cache holds them: tiles of 16 slots in MFMA operand order
 // (cache_k_index / cache_v_index), so the copy is linear and every operand read
-// from LDS is a contiguous run with no bank conflict. The next round's tiles
-// are fetched into registers while this one is multiplied.
+// from LDS is a contiguous run with no bank conflict. Tiles are fetched into
+// registers two rounds ahead and staged into one of two LDS buffers, one barrier
+// a round.
 //
 //   S^T[key][column] = K . Q^T        v_mfma_f32_16x16x32_bf16, contraction over d
 //   online softmax per column (float; running maximum, sum), once per 64 keys
@@ -58,8 +59,8 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   constexpr int NPRE = (FP_KT * DMAX / 8) / FP_THREADS;     // 16-byte chunks a thread fetches per operand
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[FP_KT * DMAX];       // 4 tiles of 16 * d
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[FP_KT * DMAX];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][FP_KT * DMAX];   // two rounds of 4 tiles of 16 * d
+  __shared__ __attribute__((aligned(16))) bf16_t Vs2[2][FP_KT * DMAX];
 
   const int tid = threadIdx.x;
   const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
@@ -114,58 +115,63 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   // step; tile tt_u of step u is the same for a whole wave, so its block id is a scalar load
   constexpr int TCH = 2 * DMAX;                  // 16-byte chunks of a tile, padded to the template's head size
   const int bs_shift = __builtin_ctz(block_size);      // block sizes are powers of two here
-  bf16x8_t kpre[NPRE], vpre[NPRE];
-  auto fetch = [&](int k0) {
+  // A fetch only issues loads, the same number every call whatever lies in range (a tile outside the
+  // visible keys reads the first visible tile instead); stage() zeroes what must not be seen as it copies
+  // the registers to LDS.
+  struct Fetched {
+    bf16x8_t kpre[NPRE], vpre[NPRE];
+  };
+  const int safe_kt = first_key & ~15;
+  auto fetch = [&](Fetched& F, int k0) {
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
       const int c = tid + u * FP_THREADS;
       const int tt = __builtin_amdgcn_readfirstlane(c / TCH), w = c % TCH;
       const int kt = k0 + tt * 16;
-      const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-      kpre[u] = zero;
-      vpre[u] = zero;
-      if (kt <= last_pos && kt + 15 >= first_key) {           // wave-uniform
-        const int blk = table[kt >> bs_shift];
-        const size_t tile_at = (((size_t)blk * Hkv + kvh) << bs_shift) * d + (size_t)((kt & (block_size - 1)) >> 4) * 16 * d;
-        if (w < 2 * d) {
-          kpre[u] = *(const bf16x8_t*)(kcache + tile_at + w * 8);
-          vpre[u] = *(const bf16x8_t*)(vcache + tile_at + w * 8);
-        }
-        // slots of the tile outside the visible range may hold anything (a freed block's bits): zero them
-        if (kt + 15 > last_pos || kt < first_key) {
-          const int kkey = kt + (w & 15);                      // K chunk w: 8 elements of slot w % 16
-          if (kkey > last_pos || kkey < first_key) kpre[u] = zero;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {                        // V chunk w: slots 4 ((w / 8) % 4) + e % 4
-            const int vkey = kt + ((w >> 3) & 3) * 4 + (e & 3);
-            if (vkey > last_pos || vkey < first_key) vpre[u][e] = (bf16_t)0.f;
-          }
-        }
-      }
+      const bool live = kt <= last_pos && kt + 15 >= first_key;         // wave-uniform
+      const int ktl = live ? kt : safe_kt;
+      const int blk = table[ktl >> bs_shift];
+      const size_t tile_at = (((size_t)blk * Hkv + kvh) << bs_shift) * d + (size_t)((ktl & (block_size - 1)) >> 4) * 16 * d;
+      const int wl = w < 2 * d ? w : 0;
+      F.kpre[u] = *(const bf16x8_t*)(kcache + tile_at + wl * 8);
+      F.vpre[u] = *(const bf16x8_t*)(vcache + tile_at + wl * 8);
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const Fetched& F, int k0, int buf) {
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
       const int c = tid + u * FP_THREADS;
       const int tt = c / TCH, w = c % TCH;
+      const int kt = k0 + tt * 16;
+      const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+      bf16x8_t kv = F.kpre[u], vv = F.vpre[u];
+      if (!(kt <= last_pos && kt + 15 >= first_key)) {
+        kv = zero;
+        vv = zero;
+      } else if (kt + 15 > last_pos || kt < first_key) {
+        // slots of the tile outside the visible range may hold anything (a freed block's bits): zero them
+        const int kkey = kt + (w & 15);                      // K chunk w: 8 elements of slot w % 16
+        if (kkey > last_pos || kkey < first_key) kv = zero;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {                        // V chunk w: slots 4 ((w / 8) % 4) + e % 4
+          const int vkey = kt + ((w >> 3) & 3) * 4 + (e & 3);
+          if (vkey > last_pos || vkey < first_key) vv[e] = (bf16_t)0.f;
+        }
+      }
       if (w < 2 * d) {
-        *(bf16x8_t*)(Ks + (tt * 2 * d + w) * 8) = kpre[u];
-        *(bf16x8_t*)(Vs + (tt * 2 * d + w) * 8) = vpre[u];
+        *(bf16x8_t*)(Ks2[buf] + (tt * 2 * d + w) * 8) = kv;
+        *(bf16x8_t*)(Vs2[buf] + (tt * 2 * d + w) * 8) = vv;
       }
     }
   };
 
-  fetch(kt_begin);
-  for (int k0 = kt_begin; k0 <= last_pos; k0 += FP_KT) {
-    __syncthreads();                       // the previous round is no longer read
-    stage();
-    __syncthreads();
-    if (k0 + FP_KT <= last_pos) fetch(k0 + FP_KT);
-
+  // one round of 64 keys from LDS buffer `buf`
+  auto compute = [&](int k0, int buf) {
+    const bf16_t* Ks = Ks2[buf];
+    const bf16_t* Vs = Vs2[buf];
     // a wave whose queries all lie before this round, or that has none, has nothing to add
-    if (w_last_pos < w_first_pos || w_last_pos < k0) continue;
-    if (window > 0 && k0 + FP_KT - 1 < w_first_pos - window + 1) continue;
+    if (w_last_pos < w_first_pos || w_last_pos < k0) return;
+    if (window > 0 && k0 + FP_KT - 1 < w_first_pos - window + 1) return;
 
     // two halves of 32 keys, each: scores, online softmax, values
 #pragma unroll
@@ -289,6 +295,27 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         }
       }
     }
+  };
+
+  // Rounds alternate between two register sets and two LDS buffers; a set is fetched two rounds
+  // ahead, right after it was staged. One barrier a round: it makes the staged tile whole, and a
+  // wave that stages buffer b for round i has passed the barrier of round i - 1, which every wave
+  // reaches only after its reads of round i - 2, the last user of buffer b.
+  Fetched F0, F1;
+  fetch(F0, kt_begin);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch(F1, kt_begin + FP_KT);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int k0 = kt_begin; k0 <= last_pos; k0 += 2 * FP_KT) {     // the bounds are the same in every thread
+    stage(F0, k0, 0);
+    __syncthreads();
+    fetch(F0, k0 + 2 * FP_KT);
+    compute(k0, 0);
+    if (k0 + FP_KT > last_pos) break;
+    stage(F1, k0 + FP_KT, 1);
+    __syncthreads();
+    fetch(F1, k0 + 3 * FP_KT);
+    compute(k0 + FP_KT, 1);
   }
 #pragma unroll
   for (int j = 0; j < NC; ++j) {
