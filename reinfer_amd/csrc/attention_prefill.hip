@@ -49,13 +49,15 @@ static FpShape fp_shape(int Hq, int Hkv, int d) {
   return s;
 }
 
-template <int DMAX, int NC>
+// EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
+template <int DMAX, int NC, bool EXACT>
 __global__ void __launch_bounds__(FP_THREADS)
 flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                      const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                      const int* __restrict__ block_tables, int max_blocks,
                      const int* __restrict__ tile_info,      // per tile: seq, first token row, n queries, first position
-                     int block_size, int Hq, int Hkv, int d, int HG, float scale_log2, int window) {
+                     int block_size, int Hq, int Hkv, int d_arg, int HG, float scale_log2, int window) {
+  const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   constexpr int NPRE = (FP_KT * DMAX / 8) / FP_THREADS;     // 16-byte chunks a thread fetches per operand
@@ -368,14 +370,20 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
   RA_CHECK(gy <= 65535, "attention_prefill: too many heads for one launch");
   dim3 grid(n_tiles, gy);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define RA_FP(DM, NCC)                                                                                \
-  flash_prefill_kernel<DM, NCC><<<grid, FP_THREADS, 0, stream>>>(                                     \
+#define RA_FP_GO(DM, NCC, EX)                                                                         \
+  flash_prefill_kernel<DM, NCC, EX><<<grid, FP_THREADS, 0, stream>>>(                                 \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, tile_info, block_size, Hq, Hkv, d, sh.hg,      \
       scale_log2, window)
+#define RA_FP(DM, NCC)                                                                                \
+  do {                                                                                                \
+    if (d == DM) RA_FP_GO(DM, NCC, true);                                                             \
+    else RA_FP_GO(DM, NCC, false);                                                                    \
+  } while (0)
   if (d <= 64) RA_FP(64, 2);
   else if (d <= 128) RA_FP(128, 2);
   else RA_FP(256, 1);
+#undef RA_FP_GO
 #undef RA_FP
   RA_LAUNCH_CHECK("attention_prefill");
   return 0;
