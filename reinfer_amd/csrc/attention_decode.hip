@@ -41,15 +41,17 @@
 
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int DMAX>
+// EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
+template <int DMAX, bool EXACT>
 __global__ void __launch_bounds__(FD_THREADS, DMAX <= 128 ? 3 : 1)
 flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                     const int* __restrict__ block_tables, int max_blocks,
                     const int* __restrict__ token_list, const int* __restrict__ seq_of_token,
-                    const int* __restrict__ positions, int block_size, int Hkv, int G, int d,
+                    const int* __restrict__ positions, int block_size, int Hkv, int G, int d_arg,
                     float scale_log2, int window, int chunk, int max_chunks, int n_tokens,
                     int t_base, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   extern __shared__ float lds[];       // [waves][G][d] outputs, then [waves][G][2] maximum and sum
@@ -342,9 +344,10 @@ static int fd_resident_workgroups(int variant, size_t lds) {
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
   hipError_t e = hipSuccess;
-  if (variant == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<64>, FD_THREADS, lds);
-  else if (variant == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<128>, FD_THREADS, lds);
-  else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<256>, FD_THREADS, lds);
+  // the exact form of a head size needs a few registers more than the other: ask for it
+  if (variant == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<64, true>, FD_THREADS, lds);
+  else if (variant == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<128, true>, FD_THREADS, lds);
+  else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<256, true>, FD_THREADS, lds);
   if (e != hipSuccess || cus <= 0 || per_cu <= 0) return 0;
   cached[variant] = cus * per_cu;
   cached_lds[variant] = lds;
@@ -392,14 +395,20 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
     float* pm = part_ml ? part_ml + rows * 2 : nullptr;
     const long items_max = (long)n * Hkv * max_chunks;
     const int grid = (int)(items_max < slots ? items_max : slots);
-#define RA_FD(DM)                                                                                     \
-  flash_decode_kernel<DM><<<grid, FD_THREADS, lds, stream>>>(                                         \
+#define RA_FD_GO(DM, EX)                                                                              \
+  flash_decode_kernel<DM, EX><<<grid, FD_THREADS, lds, stream>>>(                                     \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, list, seq_of_token, positions, block_size,     \
       Hkv, G, d, scale_log2, window, chunk, max_chunks, n, base, po, pm)
+#define RA_FD(DM)                                                                                     \
+  do {                                                                                                \
+    if (d == DM) RA_FD_GO(DM, true);                                                                  \
+    else RA_FD_GO(DM, false);                                                                         \
+  } while (0)
     if (d <= 64) RA_FD(64);
     else if (d <= 128) RA_FD(128);
     else RA_FD(256);
+#undef RA_FD_GO
 #undef RA_FD
     RA_LAUNCH_CHECK("attention_decode");
     if (max_chunks > 1) {
