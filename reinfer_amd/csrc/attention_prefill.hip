@@ -377,7 +377,7 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
       scale_log2, window)
 #define RA_FP(DM, NCC)                                                                                \
   do {                                                                                                \
-    if (d == DM) RA_FP_GO(DM, NCC, true);                                                             \
+    if (d == DM && DM <= 128) RA_FP_GO(DM, NCC, true); /* at 256 the exact form spills registers */   \
     else RA_FP_GO(DM, NCC, false);                                                                    \
   } while (0)
   if (d <= 64) RA_FP(64, 2);
