@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 9
+#define RA_ABI_VERSION 10
 
 #ifdef __cplusplus
 extern "C" {
@@ -101,10 +101,11 @@ int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const 
               const long long* seeds, const int* positions, float* scratch_val, int* scratch_idx,
               int* tokens, hipStream_t stream);
 
-// Penalties and filters on rows of float logits, in place, before ra_sample. `rows` holds one
-// record of 10 x 4 bytes per row: float temperature, top_p, min_p, repeat_penalty,
-// frequency_penalty, presence_penalty; int top_k, window_off, window_len, pad. `window` holds the
-// requests' recent tokens, row r's at [window_off, window_off + window_len).
+// Logit bias, penalties and filters on rows of float logits, in place, before ra_sample. `rows`
+// holds one record of 12 x 4 bytes per row: float temperature, top_p, min_p, repeat_penalty,
+// frequency_penalty, presence_penalty; int top_k, window_off, window_len, bias_off, bias_len, pad.
+// `window` holds the requests' recent tokens, row r's at [window_off, window_off + window_len), and
+// its logit bias as bias_len pairs (token id, float bits) from bias_off, each id once.
 int ra_filter_logits(float* logits, int n_rows, int vocab, int row_stride, const void* rows,
                      const int* window, hipStream_t stream);
 

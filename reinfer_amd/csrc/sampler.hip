@@ -169,7 +169,9 @@ __device__ __forceinline__ float filter_block_max(float v, float* red) {
 
 struct FilterRow {           // one per row, in device memory
   float temperature, top_p, min_p, repeat_penalty, frequency_penalty, presence_penalty;
-  int top_k, window_off, window_len, pad;
+  int top_k, window_off, window_len;
+  int bias_off, bias_len;      // logit bias: bias_len pairs (token id, float bits) at window[bias_off]
+  int pad;
 };
 
 __global__ void __launch_bounds__(FILTER_THREADS)
@@ -181,6 +183,18 @@ filter_logits_kernel(float* __restrict__ logits, int vocab, int row_stride, cons
   float* lg = logits + (size_t)blockIdx.x * row_stride;
   const int tid = threadIdx.x;
 
+  // additive bias per token id, before everything else (crates/cuda/kernels/sampler_kernel.cu:189-203);
+  // the caller lists every id once
+  if (fr.bias_len > 0) {
+    const int* bp = window + fr.bias_off;
+    for (int b = tid; b < fr.bias_len; b += FILTER_THREADS) {
+      const int tok = bp[2 * b];
+      if (tok < 0 || tok >= vocab) continue;
+      const float l = lg[tok];
+      if (isfinite(l)) lg[tok] = l + __int_as_float(bp[2 * b + 1]);
+    }
+    __syncthreads();
+  }
   // penalties: the first occurrence of a token in the window carries its count
   const bool pen = fr.repeat_penalty > 1.f || fr.frequency_penalty > 0.f || fr.presence_penalty > 0.f;
   if (pen && fr.window_len > 0) {

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 
 class KernelLibraryError(RuntimeError):

@@ -481,14 +481,14 @@ class HipKernels:
                      tokens.data_ptr(), _stream())
 
     def filter_logits(self, logits: torch.Tensor, params, histories) -> None:
-        """Penalties and top-k / top-p / min-p of every row's SamplingParams, in place
-        (removed tokens become -inf); ``histories[i]`` are row i's tokens so far."""
+        """Logit bias, penalties and top-k / top-p / min-p of every row's SamplingParams, in
+        place (removed tokens become -inf); ``histories[i]`` are row i's tokens so far."""
         import numpy as np
         _dev(logits)
         n, V = logits.shape
         if logits.dtype != torch.float32 or logits.stride(1) != 1:
             raise TypeError("filter_logits: logits are float32 rows")
-        rec = np.zeros((n, 10), dtype=np.float32)
+        rec = np.zeros((n, 12), dtype=np.float32)
         irec = rec.view(np.int32)
         window, off = [], 0
         for i, (p, hist) in enumerate(zip(params, histories)):
@@ -503,6 +503,14 @@ class HipKernels:
             irec[i, 7], irec[i, 8] = off, len(win)
             window += win
             off += len(win)
+            bias = getattr(p, "logit_bias", ())
+            if bias:
+                pairs = np.zeros((len(bias), 2), dtype=np.int32)
+                pairs[:, 0] = [int(t) for t, _ in bias]
+                pairs[:, 1] = np.asarray([float(b) for _, b in bias], dtype=np.float32).view(np.int32)
+                irec[i, 9], irec[i, 10] = off, len(bias)
+                window += pairs.reshape(-1).tolist()
+                off += 2 * len(bias)
         rows_t = torch.from_numpy(rec).to(logits.device)
         win_t = torch.tensor(window or [0], dtype=torch.int32).to(logits.device)
         library.call("ra_filter_logits", logits.data_ptr(), n, V, logits.stride(0), rows_t.data_ptr(),

@@ -16,6 +16,7 @@ class SamplingParams:
     frequency_penalty: Optional[float] = None   # logit -= count * penalty
     presence_penalty: Optional[float] = None    # logit -= penalty if seen
     repeat_last_n: int = 64             # penalties look at the last n tokens
+    logit_bias: Tuple[Tuple[int, float], ...] = ()      # (token id, addend to its logit), each id once
     seed: Optional[int] = None          # None: derived from the engine's seed and the arrival number
     max_tokens: int = 256               # hard cap on generated tokens
     stop_token_ids: Tuple[int, ...] = ()        # beside the model's own end-of-sequence ids
@@ -32,6 +33,15 @@ class SamplingParams:
             raise ValueError("top_p is NaN")
         if self.repeat_last_n < 0:
             raise ValueError("repeat_last_n must be >= 0")
+        # pairs (id, bias), each id once (the reference looks an id up in its sorted list,
+        # crates/cuda/src/sampler.rs:235; crates/cuda/kernels/sampler_kernel.cu:195-203)
+        pairs = tuple((int(t), float(b)) for t, b in
+                      (self.logit_bias.items() if isinstance(self.logit_bias, dict) else self.logit_bias))
+        if len({t for t, _ in pairs}) != len(pairs):
+            raise ValueError("logit_bias names a token id twice")
+        if any(t < 0 for t, _ in pairs) or any(b != b for _, b in pairs):
+            raise ValueError("logit_bias: token ids are >= 0 and biases are numbers")
+        object.__setattr__(self, "logit_bias", tuple(sorted(pairs)))
 
     @property
     def greedy(self) -> bool:
@@ -41,7 +51,7 @@ class SamplingParams:
     def filters(self) -> bool:
         """True if anything beside temperature shapes the distribution."""
         return bool((self.top_k or 0) > 0 or (self.top_p is not None and 0.0 < self.top_p < 1.0)
-                    or (self.min_p or 0.0) > 0.0 or self.penalties)
+                    or (self.min_p or 0.0) > 0.0 or self.penalties or len(self.logit_bias) > 0)
 
     @property
     def penalties(self) -> bool:

@@ -179,7 +179,7 @@ class KernelDouble:
                 logits[i], max(0.0, p.temperature), top_k=p.top_k or 0, top_p=p.top_p or 0.0,
                 min_p=p.min_p or 0.0, repeat_penalty=p.repeat_penalty or 0.0,
                 frequency_penalty=p.frequency_penalty or 0.0, presence_penalty=p.presence_penalty or 0.0,
-                window=win).float()
+                window=win, logit_bias=p.logit_bias).float()
 
     def sample(self, logits, temperature, seeds, positions, tokens):
         from plain_qwen3 import mix64, splitmix64, unit_from_u64

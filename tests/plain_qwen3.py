@@ -207,8 +207,12 @@ def unit_from_u64(x: int) -> float:
 
 def filter_logits(logits: torch.Tensor, temperature: float, *, top_k: int = 0, top_p: float = 0.0,
                   min_p: float = 0.0, repeat_penalty: float = 0.0, frequency_penalty: float = 0.0,
-                  presence_penalty: float = 0.0, window: Sequence[int] = ()) -> torch.Tensor:
-    """Penalties, then the filters on softmax(logits / T); removed tokens are -inf.
+                  presence_penalty: float = 0.0, window: Sequence[int] = (),
+                  logit_bias: Sequence = ()) -> torch.Tensor:
+    """Logit bias, penalties, then the filters on softmax(logits / T); removed tokens are -inf.
+
+    Bias (crates/cuda/kernels/sampler_kernel.cu:189-203): logit[id] += bias for the
+    listed ids, before anything else; a logit that is not finite stays as it is.
 
     Penalties (crates/cuda/kernels/sampler_kernel.cu:207-221): for a token that
     occurs cnt > 0 times in the window, logit -= cnt * freq + pres, then logit > 0
@@ -220,6 +224,9 @@ def filter_logits(logits: torch.Tensor, temperature: float, *, top_k: int = 0, t
     """
     l = logits.clone().double()
     V = l.numel()
+    for t, b in logit_bias:
+        if 0 <= t < V and torch.isfinite(l[t]):
+            l[t] = l[t] + float(torch.tensor(b, dtype=torch.float32))
     if window and (repeat_penalty > 1 or frequency_penalty > 0 or presence_penalty > 0):
         counts: Dict[int, int] = {}
         for t in window:

@@ -414,6 +414,9 @@ def test_filter_logits_against_plain(V):
         dict(temperature=1.0, repeat_penalty=1.3, frequency_penalty=0.4, presence_penalty=0.2, top_k=7),
         dict(temperature=0.0, repeat_penalty=1.5, top_k=3),          # greedy: penalties only
         dict(temperature=1.0, top_k=1),
+        # a bias lifts an unlikely token over the favourite and sinks the favourite; with penalties and a filter
+        dict(temperature=0.0, logit_bias=((3, 40.0), (int(base.argmax()), -50.0))),
+        dict(temperature=0.8, logit_bias=((5, 25.0), (999, -3.5), (0, 1.25)), top_k=4, frequency_penalty=0.3),
     ]
     hist = torch.randint(0, V, (90,), generator=g).tolist()
     hist += hist[:10] + [int(base.argmax())] * 3                    # repeats, and the favourite three times
@@ -427,6 +430,8 @@ def test_filter_logits_against_plain(V):
             row[17] = float("-inf")
         kw = {k: v for k, v in c.items() if k != "temperature"}
         ref = plain.filter_logits(row, c["temperature"], window=hist[-64:], **kw)
+        if i == 7:
+            assert int(ref.argmax()) == 3                                # the bias decides the greedy token
         got = logits[i].cpu().double()
         kept_ref, kept_got = torch.isfinite(ref), torch.isfinite(got)
         if i == 0:

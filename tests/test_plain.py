@@ -126,3 +126,18 @@ def test_splitmix_vectors_and_greedy_ties():
     assert plain.splitmix64(1) == 0x910A2DEC89025CC1
     assert plain.unit_from_u64((1 << 64) - 1) < 1.0 and plain.unit_from_u64(0) == 0.0
     assert plain.argmax_first(torch.tensor([1.0, 5.0, 5.0, 2.0])) == 1      # first maximum
+
+
+def test_logit_bias_is_added_first_and_validated():
+    """Reference semantics (crates/cuda/tests/sampler_gpu.rs:369-372): a bias of -5 on the
+    favourite flips the greedy token to the runner-up; non-finite logits stay."""
+    import pytest
+    from reinfer_amd.sampling import SamplingParams
+    logits = torch.tensor([0.0, 2.0, 3.0, float("-inf")])
+    out = plain.filter_logits(logits, 0.0, logit_bias=((2, -5.0), (3, 100.0)))
+    assert int(out.argmax()) == 1 and out[3] == float("-inf") and out[2] == -2.0
+    p = SamplingParams(logit_bias={7: 1.5, 2: -1.0})
+    assert p.logit_bias == ((2, -1.0), (7, 1.5)) and p.filters
+    with pytest.raises(ValueError, match="twice"):
+        SamplingParams(logit_bias=((1, 0.5), (1, 0.25)))
+    assert not SamplingParams().filters
