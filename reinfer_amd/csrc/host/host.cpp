@@ -561,6 +561,7 @@ struct Request {
   float temperature = 0.f;
   int64_t seed64 = 0;              // the seed's low 64 bits as the kernels take them
   std::vector<int> stop_ids;
+  std::vector<std::vector<int>> stop_seqs;       // token sequences that end the request
 
   int num_tokens() const { return (int)(prompt.size() + output.size()); }
   int remaining() const { return num_tokens() - num_computed; }
@@ -655,6 +656,11 @@ struct Scheduler {
     req->filters = params.attr("filters").cast<bool>();
     req->temperature = std::max(0.f, params.attr("temperature").cast<float>());
     for (auto t : params.attr("stop_token_ids")) req->stop_ids.push_back(t.cast<int>());
+    for (auto seq : params.attr("stop_sequences")) {
+      std::vector<int> v;
+      for (auto t : seq) v.push_back(t.cast<int>());
+      if (!v.empty()) req->stop_seqs.push_back(std::move(v));      // an empty pattern never matches
+    }
     requests[rid] = req;
     waiting.push_back(req);
     return req;
@@ -818,7 +824,19 @@ struct Scheduler {
       if (next >= tokens.size()) throw py::value_error("complete: fewer tokens than portions that sample");
       const int tok = tokens[next++];
       const bool is_eos = std::find(eos.begin(), eos.end(), tok) != eos.end();
-      const bool stop = (is_eos && !r->ignore_eos) ||
+      // A stop sequence fires the moment it is a suffix of the generated stream; its last token is
+      // consumed like a stop id, the ones before it were emitted (crates/scheduler/src/stop.rs:1-12,
+      // req.rs:281-300).
+      bool seq_stop = false;
+      for (auto& pat : r->stop_seqs) {
+        const size_t L = pat.size();
+        if (tok != pat[L - 1] || r->output.size() + 1 < L) continue;
+        if (std::equal(pat.begin(), pat.end() - 1, r->output.end() - (L - 1))) {
+          seq_stop = true;
+          break;
+        }
+      }
+      const bool stop = seq_stop || (is_eos && !r->ignore_eos) ||
                         std::find(r->stop_ids.begin(), r->stop_ids.end(), tok) != r->stop_ids.end();
       if (stop) {
         r->finish_reason = py::str("stop");

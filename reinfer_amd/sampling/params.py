@@ -20,6 +20,7 @@ class SamplingParams:
     seed: Optional[int] = None          # None: derived from the engine's seed and the arrival number
     max_tokens: int = 256               # hard cap on generated tokens
     stop_token_ids: Tuple[int, ...] = ()        # beside the model's own end-of-sequence ids
+    stop_sequences: Tuple[Tuple[int, ...], ...] = ()    # token sequences that end the request when generated
     ignore_eos: bool = False
 
     def __post_init__(self):
@@ -42,6 +43,10 @@ class SamplingParams:
         if any(t < 0 for t, _ in pairs) or any(b != b for _, b in pairs):
             raise ValueError("logit_bias: token ids are >= 0 and biases are numbers")
         object.__setattr__(self, "logit_bias", tuple(sorted(pairs)))
+        # stop strings arrive as token-id sequences (the text belongs to the layer above,
+        # crates/scheduler/src/stop.rs:1-6); empty ones are ignored
+        object.__setattr__(self, "stop_sequences",
+                           tuple(tuple(int(t) for t in seq) for seq in self.stop_sequences if len(seq) > 0))
 
     @property
     def greedy(self) -> bool:

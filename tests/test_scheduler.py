@@ -226,3 +226,23 @@ def test_replay_twice_is_identical():
         return log, outs
     for seed in range(5):
         assert run(seed) == run(seed)
+
+
+def test_stop_sequences_fire_on_the_generated_suffix():
+    """The reference's matcher cases (crates/scheduler/src/stop.rs:97-158) through the scheduler:
+    a pattern spanning steps, a mismatch that resets, 'aaa' on a stream of a's, overlapping
+    patterns, an empty pattern. The last token of the match is consumed, the ones before it
+    were emitted; the prompt is no part of the stream."""
+    def run(stream, patterns, prompt=(1,)):
+        m, s = make()
+        s.add("a", list(prompt), SamplingParams(max_tokens=50, ignore_eos=True, stop_sequences=patterns), seed=0)
+        it = iter(stream)
+        return drive(m, s, token_fn=lambda rid, pos: next(it))["a"]
+    assert run([1, 7, 9], ((7,),)) == ([1], "stop")
+    assert run([3, 1, 9, 3, 1, 4, 8], ((3, 1, 4),)) == ([3, 1, 9, 3, 1], "stop")
+    assert run([1, 2, 1, 3, 1, 2, 1, 2, 5], ((1, 2, 1, 2),)) == ([1, 2, 1, 3, 1, 2, 1], "stop")
+    assert run([5, 5, 5, 5], ((5, 5, 5),)) == ([5, 5], "stop")
+    assert run([1, 2, 3, 4], ((1, 2, 3), (2, 3))) == ([1, 2], "stop")
+    assert run([6, 4, 2], ((), (4,))) == ([6], "stop")
+    # the prompt's tokens do not count: 3 1 in the prompt, 4 generated first
+    assert run([4, 3, 1, 4, 0], ((3, 1, 4),), prompt=(3, 1)) == ([4, 3, 1], "stop")
