@@ -65,7 +65,8 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   __shared__ __attribute__((aligned(16))) bf16_t Vs2[2][FP_KT * DMAX];
 
   const int tid = threadIdx.x;
-  const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
+  const int lane = tid & (RA_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / RA_WAVE);      // scalar: tests on it are branches
   const int r = lane & 15, g = lane >> 4;
   const int G = Hq / Hkv;
   const int n_hgrp = G / HG;
@@ -98,7 +99,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   float m[NC], l[NC];
 #pragma unroll
   for (int j = 0; j < NC; ++j) {
-    m[j] = -INFINITY;
+    m[j] = q_live[j] ? -INFINITY : 0.f;      // a column without a query adds zeros and never asks for a new maximum
     l[j] = 0.f;
 #pragma unroll
     for (int i = 0; i < NOT; ++i) acc[j][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -162,7 +163,11 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
       }
       if (w < 2 * d) {
         *(bf16x8_t*)(Ks2[buf] + (tt * 2 * d + w) * 8) = kv;
-        *(bf16x8_t*)(Vs2[buf] + (tt * 2 * d + w) * 8) = vv;
+        // V: the two tiles of a half interleaved in runs of 8 bytes, so that an operand of the output
+        // product (4 slots of the first tile, 4 of the second) is one 16-byte read
+        bf16_t* vd = Vs2[buf] + ((tt >> 1) * 4 * d + 2 * w) * 8 + (tt & 1) * 4;
+        *(bf16x4_t*)(vd) = (bf16x4_t){vv[0], vv[1], vv[2], vv[3]};
+        *(bf16x4_t*)(vd + 8) = (bf16x4_t){vv[4], vv[5], vv[6], vv[7]};
       }
     }
   };
@@ -191,22 +196,18 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         const int e = dt * 32 + g * 8;
         return (e < d) ? *(const bf16x8_t*)(Ks + (kp * 2 + ks) * 16 * d + ((dt * 4 + g) * 16 + r) * 8) : zero8;
       };
-      auto v_operand = [&](int ot, int hi) -> bf16x4_t {
-        const bf16_t* v0 = Vs + (2 * kp + hi) * 16 * d + ((ot * 4 + g) * 16 + r) * 4;
-        return (ot * 16 < d) ? *(const bf16x4_t*)(v0) : (bf16x4_t){0, 0, 0, 0};
+      auto v_operand = [&](int ot) -> bf16x8_t {
+        return (ot * 16 < d) ? *(const bf16x8_t*)(Vs + (kp * 4 * d + (ot * 4 + g) * 16 + r) * 8) : zero8;
       };
       bf16x8_t ka[AHEAD ? 2 : 1][AHEAD ? NDT : 1];
-      bf16x4_t vlo[AHEAD ? NOT : 1], vhi[AHEAD ? NOT : 1];
+      bf16x8_t va[AHEAD ? NOT : 1];
       if constexpr (AHEAD) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
           for (int dt = 0; dt < NDT; ++dt) ka[ks][dt] = k_operand(ks, dt);
 #pragma unroll
-        for (int ot = 0; ot < NOT; ++ot) {
-          vlo[ot] = v_operand(ot, 0);
-          vhi[ot] = v_operand(ot, 1);
-        }
+        for (int ot = 0; ot < NOT; ++ot) va[ot] = v_operand(ot);
         __builtin_amdgcn_sched_barrier(0);     // the reads stay ahead of the products
       }
       // scores S^T[key][column] for 2 sub-tiles of 16 keys
@@ -244,17 +245,30 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
               if (!(q_live[j] && key <= q_pos && key >= q_lo)) s[ks][j][i] = -INFINITY;
             }
         }
-        float tmax = fmaxf(fmaxf(fmaxf(s[0][j][0], s[0][j][1]), fmaxf(s[0][j][2], s[0][j][3])),
-                           fmaxf(fmaxf(s[1][j][0], s[1][j][1]), fmaxf(s[1][j][2], s[1][j][3])));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE));
-        tmax *= scale_log2;                              // the scale is positive: it commutes with the maximum
-        // The running maximum follows the true one only when that has grown by more than 2^8:
-        // until then the probabilities are at most 256 times larger than with the true maximum,
-        // which float sums and bfloat16 operands hold as well, and the accumulators need no rescaling.
-        // The wave decides as a whole, so the rare rescaling is a uniform branch.
-        const bool grow = tmax > m[j] + 8.f;             // false for -inf maxima
-        if (__any(grow)) {
+        // Probabilities against the running maximum m first; m follows the true maximum only when
+        // some probability comes out above 2^8 (the true maximum has grown by more than 8 in the
+        // exponent): until then float sums and bfloat16 operands hold the larger values as well, and
+        // the accumulators need no rescaling. A lane tests the 8 values it holds itself; the exchange
+        // between lanes that finds a column's maximum is left to the rare branch, which the wave
+        // takes as a whole, for every column: it rescales and computes the probabilities again. A
+        // column that has seen no key yet (m = -inf) always takes it, so m never stays unset while
+        // keys are visible.
+        float p[8];
+        auto probabilities = [&]() {
+          const float base = (m[j] == -INFINITY) ? 0.f : m[j];
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              p[ks * 4 + i] = fp_exp2(fmaf(s[ks][j][i], scale_log2, -base));      // masked: exp2(-inf) = 0
+        };
+        probabilities();
+        const float big = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+        if (__any(!(big <= 256.f) || m[j] == -INFINITY)) {           // an overflowed or undefined value counts as large
+          float tmax = fmaxf(fmaxf(fmaxf(s[0][j][0], s[0][j][1]), fmaxf(s[0][j][2], s[0][j][3])),
+                             fmaxf(fmaxf(s[1][j][0], s[1][j][1]), fmaxf(s[1][j][2], s[1][j][3])));
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 16, RA_WAVE));
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 32, RA_WAVE)) * scale_log2;    // the scale is positive
           const float mn = fmaxf(m[j], tmax);
           // a column with nothing visible so far keeps m = -inf and adds zeros
           const float corr = (mn == -INFINITY) ? 1.f : fp_exp2(m[j] - mn);
@@ -264,17 +278,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
           for (int ot = 0; ot < NOT; ++ot)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[j][ot][i] *= corr;
+          probabilities();
         }
-        const float base = (m[j] == -INFINITY) ? 0.f : m[j];
         float psum = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float p = fp_exp2(fmaf(s[ks][j][i], scale_log2, -base));      // masked: exp2(-inf) = 0
-            psum += p;
-            pb[j][ks * 4 + i] = from_f32<bf16_t>(p);
-          }
+        for (int e = 0; e < 8; ++e) {
+          psum += p[e];
+          pb[j][e] = from_f32<bf16_t>(p[e]);
+        }
         l[j] += psum;
       }
       // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
@@ -282,15 +293,9 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
       for (int ot = 0; ot < NOT; ++ot) {
         if (ot * 16 < d) {
-          bf16x4_t lo4, hi4;
-          if constexpr (AHEAD) {
-            lo4 = vlo[ot];
-            hi4 = vhi[ot];
-          } else {
-            lo4 = v_operand(ot, 0);
-            hi4 = v_operand(ot, 1);
-          }
-          const bf16x8_t a = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+          bf16x8_t a;
+          if constexpr (AHEAD) a = va[ot];
+          else a = v_operand(ot);
 #pragma unroll
           for (int j = 0; j < NC; ++j)
             acc[j][ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[j], acc[j][ot], 0, 0, 0);
