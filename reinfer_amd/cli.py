@@ -21,8 +21,18 @@ import time
 from typing import List, Optional
 
 
+def _backend(name: str) -> str:
+    """``--backend`` as the reference parses it (bin/reinfer/src/main.rs:80-90): a known name or an
+    error that lists the names. Only ``auto`` and ``hip`` exist here."""
+    if name in ("auto", "hip"):
+        return name
+    raise argparse.ArgumentTypeError(f"unknown backend '{name}' (auto|hip)")
+
+
 def _add_run_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("model", help="model folder (config.json + model.safetensors)")
+    p.add_argument("--backend", type=_backend, default="auto", metavar="BACKEND",
+                   help="auto|hip: this engine has one backend, the MI355X (main.rs:252 names auto|cuda|ascend|cpu)")
     p.add_argument("-n", dest="max_tokens", type=int, default=256, metavar="MAX_TOKENS",
                    help="max new tokens (hard cap)")
     p.add_argument("-t", dest="temperature", type=float, default=1.0, metavar="TEMP",

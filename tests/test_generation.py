@@ -120,3 +120,15 @@ def test_command_line_run(tmp_path):
     assert r.returncode == 0, r.stderr
     assert [int(t) for t in r.stdout.split()] == want
     assert "PERF " in r.stderr and "tok_s=" in r.stderr and "first_token_ms=" in r.stderr
+
+
+def test_command_line_backend_option():
+    """`run m --backend bogus` is a usage error and the default is auto
+    (bin/reinfer/src/main.rs:2135-2140); here the only backends are auto and hip."""
+    from reinfer_amd import cli
+    with pytest.raises(SystemExit) as e:
+        cli.main(["run", "m", "--backend", "bogus"])
+    assert e.value.code == 2
+    with pytest.raises(SystemExit):
+        cli.main(["run", "m", "--backend", "cuda"])
+    assert cli._backend("auto") == "auto" and cli._backend("hip") == "hip"
