@@ -231,10 +231,9 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
       // keys strictly inside every query's view need no mask
       const bool inner = kh + 31 <= w_first_pos && w_qend <= nq &&
                          (window <= 0 || kh >= w_last_pos - window + 1);
-      bf16x8_t pb[NC];
+      if (!inner) {
 #pragma unroll
-      for (int j = 0; j < NC; ++j) {
-        if (!inner) {
+        for (int j = 0; j < NC; ++j) {
           const int q_pos = pos0 + qi[j];
           const int q_lo = (window > 0 && q_pos - window + 1 > 0) ? q_pos - window + 1 : 0;
 #pragma unroll
@@ -245,6 +244,11 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
               if (!(q_live[j] && key <= q_pos && key >= q_lo)) s[ks][j][i] = -INFINITY;
             }
         }
+      }
+      // Column tile by column tile: probabilities, then at once the tile's output products, so that the
+      // matrix core works on them while the next tile's probabilities are computed.
+#pragma unroll
+      for (int j = 0; j < NC; ++j) {
         // Probabilities against the running maximum m first; m follows the true maximum only when
         // some probability comes out above 2^8 (the true maximum has grown by more than 8 in the
         // exponent): until then float sums and bfloat16 operands hold the larger values as well, and
@@ -281,24 +285,32 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
           probabilities();
         }
         float psum = 0.f;
+        bf16x8_t pb;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           psum += p[e];
-          pb[j][e] = from_f32<bf16_t>(p[e]);
+          pb[e] = from_f32<bf16_t>(p[e]);
         }
         l[j] += psum;
-      }
-      // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
-      // k-slots (g, e): e < 4 -> key 4g + e of the first 16-key tile, e >= 4 -> of the second
+        // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
+        // k-slots (g, e): e < 4 -> key 4g + e of the first 16-key tile, e >= 4 -> of the second
 #pragma unroll
-      for (int ot = 0; ot < NOT; ++ot) {
-        if (ot * 16 < d) {
-          bf16x8_t a;
-          if constexpr (AHEAD) a = va[ot];
-          else a = v_operand(ot);
+        for (int ot = 0; ot < NOT; ++ot) {
+          if (ot * 16 < d) {
+            bf16x8_t a;
+            if constexpr (AHEAD) a = va[ot];
+            else a = v_operand(ot);
+            acc[j][ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[j][ot], 0, 0, 0);
+          }
+        }
+        if (j + 1 < NC) {
+          // one product, then three of the next tile's vector instructions, and so on: a wave issues
+          // in order, so only alternating them lets the two kinds of work overlap
 #pragma unroll
-          for (int j = 0; j < NC; ++j)
-            acc[j][ot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[j], acc[j][ot], 0, 0, 0);
+          for (int ot = 0; ot < NOT; ++ot) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);     // VALU
+          }
         }
       }
     }
