@@ -41,6 +41,26 @@
 
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// How one token's keys [lo, p] are cut: into at most max_chunks chunks of equal length, a multiple of
+// 128 and at least chunk_min (a power of two; but for the rounding), from the 16-key tile that holds lo. Equal chunks of
+// the token's own length, not of the longest context in the batch: no work item is a short remainder.
+struct FdCut {
+  int base;    // first key of chunk 0 (a multiple of 16)
+  int chunk;   // keys of a chunk
+  int n;       // chunks
+};
+__device__ __forceinline__ FdCut fd_cut(int p, int lo, int chunk_shift, int max_chunks) {
+  FdCut c;
+  c.base = lo & ~15;
+  const int span = p - c.base + 1;
+  int want = (span + (1 << chunk_shift) - 1) >> chunk_shift;       // chunk_min = 1 << chunk_shift
+  want = want < max_chunks ? want : max_chunks;
+  c.chunk = ((span + want - 1) / want + 127) & ~127;
+  c.n = want;                                                      // fewer if the rounding up to 128 covers the keys sooner
+  while ((c.n - 1) * c.chunk >= span) --c.n;
+  return c;
+}
+
 // EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
 template <int DMAX, bool EXACT>
 __global__ void __launch_bounds__(FD_THREADS, DMAX <= 128 ? 3 : 1)
@@ -49,7 +69,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
                     const int* __restrict__ block_tables, int max_blocks,
                     const int* __restrict__ token_list, const int* __restrict__ seq_of_token,
                     const int* __restrict__ positions, int block_size, int Hkv, int G, int d_arg,
-                    float scale_log2, int window, int chunk, int max_chunks, int n_tokens,
+                    float scale_log2, int window, int chunk_shift, int max_chunks, int n_tokens,
                     int t_base, float* __restrict__ part_o, float* __restrict__ part_ml) {
   const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
@@ -66,7 +86,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
   for (int i = tid; i < n_tokens; i += FD_THREADS) {
     const int pi = positions[token_list ? token_list[i] : t_base + i];
     const int loi = (window > 0 && pi - window + 1 > 0) ? pi - window + 1 : 0;
-    first_item[i + 1] = pi / chunk - loi / chunk + 1;
+    first_item[i + 1] = fd_cut(pi, loi, chunk_shift, max_chunks).n;
   }
   if (tid == 0) first_item[0] = 0;
   __syncthreads();
@@ -99,9 +119,9 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     const int t = token_list ? token_list[li] : t_base + li;
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int c_first = lo / chunk, c_last = p / chunk;
-    const int ci = c_first + (slot - first_item[li]);
-    const int n_chunks = c_last - c_first + 1;
+    const FdCut cut = fd_cut(p, lo, chunk_shift, max_chunks);
+    const int ci = slot - first_item[li];
+    const int n_chunks = cut.n;
     const int seq = seq_of_token[t];
     const int* table = block_tables + (size_t)seq * max_blocks;
     const int Hq = Hkv * G;
@@ -119,8 +139,8 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     for (int i = 0; i < NOT; ++i) acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    const int k_begin = ci * chunk;
-    const int k_end = min(k_begin + chunk, p + 1);
+    const int k_begin = cut.base + ci * cut.chunk;
+    const int k_end = min(k_begin + cut.chunk, p + 1);
     // Block ids come through the scalar cache (the index is made uniform for the compiler) and are asked
     // for one step ahead: a vector load would queue behind the K and V loads in flight, and under load a
     // load that the K and V loads depend on costs microseconds.
@@ -245,7 +265,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     }
     __syncthreads();
     const size_t pair = (size_t)li * Hkv + kvh;
-    const size_t prow = (pair * max_chunks + (ci - c_first)) * G;      // [pair][chunk][head]
+    const size_t prow = (pair * max_chunks + ci) * G;      // [pair][chunk][head]
     for (int idx = tid; idx < G * d; idx += FD_THREADS) {
       const int h = idx / d, e = idx % d;
       float mw = -INFINITY;
@@ -278,13 +298,13 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
 __global__ void __launch_bounds__(RA_WAVE)
 flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                           bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
-                          const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk,
+                          const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk_shift,
                           int max_chunks, int t_base) {
   const int head = blockIdx.x, li = blockIdx.y;
   const int t = token_list ? token_list[li] : t_base + li;
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int n_chunks = p / chunk - lo / chunk + 1;
+  const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks).n;
   if (n_chunks == 1) return;                           // written by the first kernel
   const int lane = threadIdx.x;
   const int kvh = head / G, h = head % G;
@@ -362,6 +382,16 @@ extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_si
           block_size % 16 == 0) ? 1 : 0;
 }
 
+// Workgroups of the decode kernel that the current device holds at once for these sizes (its grid); 0 if
+// the sizes are not taken or the device cannot be asked. The caller cuts the keys so that the work items
+// fill this grid once.
+extern "C" int ra_attention_decode_slots(int Hq, int Hkv, int d) {
+  if (!ra_attention_decode_supports(Hq, Hkv, d, 16)) return 0;
+  const size_t lds = (size_t)FD_WAVES * (Hq / Hkv) * (d + 2) * sizeof(float);
+  if (lds > 64 * 1024) return 0;
+  return fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, lds);
+}
+
 extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride,
                                    const void* kcache, const void* vcache, const int* block_tables,
                                    int max_blocks, const int* token_list, const int* seq_of_token,
@@ -373,7 +403,8 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
            "attention_decode: unsupported sizes (%d query heads, %d KV heads, head size %d, block %d)", Hq,
            Hkv, d, block_size);
   RA_CHECK(max_blocks > 0 && window >= 0, "attention_decode: bad cache geometry");
-  RA_CHECK(chunk >= 128 && chunk % 128 == 0, "attention_decode: chunk %d is no multiple of 128", chunk);
+  RA_CHECK(chunk >= 128 && (chunk & (chunk - 1)) == 0, "attention_decode: chunk %d is no power of two from 128", chunk);
+  const int chunk_shift = __builtin_ctz((unsigned)chunk);
   RA_CHECK(max_chunks >= 1 && max_chunks <= 65535, "attention_decode: %d chunks outside 1..65535", max_chunks);
   RA_CHECK(max_chunks == 1 || (part_o && part_ml),
            "attention_decode: more than one chunk needs the partial buffers");
@@ -399,7 +430,7 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   flash_decode_kernel<DM, EX><<<grid, FD_THREADS, lds, stream>>>(                                     \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, list, seq_of_token, positions, block_size,     \
-      Hkv, G, d, scale_log2, window, chunk, max_chunks, n, base, po, pm)
+      Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n, base, po, pm)
 #define RA_FD(DM)                                                                                     \
   do {                                                                                                \
     if (d == DM) RA_FD_GO(DM, true);                                                                  \
@@ -414,7 +445,7 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
     if (max_chunks > 1) {
       dim3 mg(Hq, n);
       flash_decode_merge_kernel<<<mg, RA_WAVE, 0, stream>>>(po, pm, (bf16_t*)out, out_stride, list, positions,
-                                                           Hkv, G, d, window, chunk, max_chunks, base);
+                                                           Hkv, G, d, window, chunk_shift, max_chunks, base);
       RA_LAUNCH_CHECK("attention_decode merge");
     }
   }

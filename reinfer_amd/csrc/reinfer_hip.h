@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 10
+#define RA_ABI_VERSION 11
 
 #ifdef __cplusplus
 extern "C" {
@@ -77,10 +77,12 @@ int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C,
 // in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);
 // block_size and d are multiples of 16.
 //
-// bfloat16 flash-decode: one query per listed token; keys in chunks of `chunk` (a multiple of
-// 128), max_chunks = chunks of the longest context. With more than one chunk: part_o float
-// [n_tokens * Hkv, max_chunks, G, d], part_ml float [.., 2], merged by a second kernel.
+// bfloat16 flash-decode: one query per listed token. A token's keys are cut into equal chunks of its
+// own length: at most max_chunks of them, each a multiple of 128 and about `chunk` (a power of two, 128 or
+// more) or longer. With max_chunks > 1: part_o float [n_tokens * Hkv, max_chunks, G, d], part_ml float
+// [.., 2], merged by a second kernel.
 int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size);
+int ra_attention_decode_slots(int Hq, int Hkv, int d);   // workgroups of its grid on this device (0: unknown)
 int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                         const void* vcache, const int* block_tables, int max_blocks,
                         const int* token_list, const int* seq_of_token, const int* positions,

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 class KernelLibraryError(RuntimeError):
@@ -69,6 +69,8 @@ def load() -> ctypes.CDLL:
         for name in ("ra_attention_decode_supports", "ra_attention_prefill_supports"):
             getattr(lib, name).restype = c_int
             getattr(lib, name).argtypes = [c_int, c_int, c_int, c_int]
+        lib.ra_attention_decode_slots.restype = c_int
+        lib.ra_attention_decode_slots.argtypes = [c_int, c_int, c_int]
         lib.ra_attention_prefill_tile.restype = c_int
         lib.ra_attention_prefill_tile.argtypes = [c_int, c_int, c_int]
         lib.ra_gemm_skinny_max_rows.restype = c_int
