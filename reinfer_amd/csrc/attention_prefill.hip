@@ -1,24 +1,28 @@
 // Paged flash attention for prompt portions, bfloat16, on the matrix cores.
 //
-// A workgroup (8 waves, two a SIMD, so one wave's softmax arithmetic overlaps
-// the other's matrix products) takes one tile of consecutive query tokens of
+// A workgroup (8 waves, two a SIMD) takes one tile of consecutive query tokens of
 // one request and HG query heads that share a KV head: 8 * NC column tiles of
 // 16 columns, tile c = run c / HG of 16 queries, head c % HG; a wave owns NC
 // adjacent column tiles, so every key and value it reads from LDS feeds NC
 // MFMAs and all waves share one staged copy. Keys and values come from the
 // request's block table, earlier context and the portion's own tokens alike
 // (they were stored before this kernel runs), 64 keys a round, copied to LDS
-// as the cache holds them: tiles of 16 slots in MFMA operand order
-// (cache_k_index / cache_v_index), so the copy is linear and every operand read
-// from LDS is a contiguous run with no bank conflict. Tiles are fetched into
-// registers two rounds ahead and staged into one of two LDS buffers, one barrier
-// a round.
+// tile by tile of 16 slots in the cache's MFMA operand order (cache_k_index /
+// cache_v_index; V with the two tiles of a 32-key half interleaved in runs of 8
+// bytes), so every operand read from LDS is one contiguous 16-byte run a lane with
+// no bank conflict. Tiles are fetched into registers two rounds ahead and staged
+// into one of two LDS buffers, one barrier a round.
 //
 //   S^T[key][column] = K . Q^T        v_mfma_f32_16x16x32_bf16, contraction over d
-//   online softmax per column (float; running maximum, sum), once per 64 keys
+//   online softmax per column (float; running maximum, sum), once per 32 keys
 //   O^T[d][column]  += V^T . P        contraction over 32 keys; the probabilities
 //                                     are the MFMA's second operand straight from
 //                                     the score registers (two score tiles packed)
+//
+// The parts of a round run one after the other in a wave, and the two waves of a
+// SIMD overlap little (timed with parts left out); what a wave's own instruction
+// stream alternates overlaps: a column tile's output products with the next
+// tile's exponentials.
 //
 // Causal: a query at position p sees keys <= p (and > p - window if a window is
 // set). The reference's prompt attention is a vendored library kernel that sees
