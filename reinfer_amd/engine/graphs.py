@@ -27,7 +27,7 @@ from .. import kernels
 from .._hostlib import host as host_runtime
 from .batch import StepBatch, StepEntry
 
-MAX_GRAPH_BATCH = 64
+MAX_GRAPH_BATCH = 128
 
 
 def _bucket(n: int) -> int:
@@ -35,6 +35,12 @@ def _bucket(n: int) -> int:
     while b < n:
         b *= 2
     return b
+
+
+def _batch_bucket(n: int) -> int:
+    """Rows a captured step is padded to: powers of two up to 64, from there multiples of 16 (a
+    product's time grows with its rows once it has that many, and so would the padding's cost)."""
+    return _bucket(n) if n <= 64 else -(-n // 16) * 16
 
 
 class _CapturedStep:
@@ -145,7 +151,7 @@ class DecodeGraphs:
         context after it. -> (logits [B_pad, vocab] static, tokens [B_pad] static): rows past the
         entries are padding; both are overwritten by the next replay of this bucket."""
         r = self.runner
-        B = _bucket(len(entries))
+        B = _batch_bucket(len(entries))
         ctx_cap = max(256, _bucket(longest))
         ctx_cap = min(ctx_cap, max(256, _bucket(r.max_model_len)))
         key = (B, ctx_cap)

@@ -49,6 +49,7 @@ class ModelRunner:
         self.device = device
         self.block_size = int(block_size)
         self.max_model_len = min(max_model_len or spec.max_positions, spec.max_positions)
+        self.max_seqs = int(max_seqs)
         self.model = DecoderModel(spec, weights, dtype, device)
         needs = self.model.cache_needs()
 
@@ -149,8 +150,8 @@ class ModelRunner:
         free, total = torch.cuda.mem_get_info(self.device)
         usable = free - (1.0 - fraction) * total
         blocks = int(usable // per_block)
-        # no request can hold more than max_model_len tokens; 64 requests is the cap on live ones
-        cap = 64 * (-(-self.max_model_len // self.block_size))
+        # no request can hold more than max_model_len tokens, and max_seqs requests are live at most
+        cap = self.max_seqs * (-(-self.max_model_len // self.block_size))
         return max(1, min(blocks, cap))
 
     # ----------------------------------------------------------- requests

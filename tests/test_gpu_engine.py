@@ -140,3 +140,55 @@ def test_batch_order_does_not_matter(folders):
     for r in seqs:
         assert rel_err(a[r], alone[r]) < 1e-5
         assert rel_err(b[r], alone[r]) < 1e-5
+
+
+@pytest.mark.parametrize("which,n_req", [("A", 5), ("B", 70)])
+def test_decode_graphs_replay_like_eager_steps(folders, which, n_req):
+    """Decode steps replay captured HIP graphs (one per batch-size and context bucket, library
+    products included above 64 rows). Every replay is checked against a runner that launches the
+    same step kernel by kernel: the same bucket several times, with prompt steps (eager work and
+    synchronisations) between the replays, requests leaving, and a second context bucket."""
+    dtype = "bfloat16"
+    V = vocab(which)
+    with_graphs = runner_for(folders, which, dtype, max_tokens=n_req * 320, max_seqs=128)
+    eager = runner_for(folders, which, dtype, max_tokens=n_req * 320, max_seqs=128, use_graphs=False)
+    assert with_graphs.graphs is not None and eager.graphs is None
+    seqs = {f"r{i}": random_tokens(300, V, 100 + i) for i in range(n_req)}
+    fed = {r: 0 for r in seqs}
+
+    def both(items):
+        outs = []
+        for runner in (with_graphs, eager):
+            entries = []
+            for r, n in items:
+                if not runner.has_request(r):
+                    runner.add_request(r)
+                entries.append(StepEntry(r, list(seqs[r][fed[r]:fed[r] + n]), [n - 1]))
+            outs.append(runner.step(entries).float().cpu())
+        for r, n in items:
+            fed[r] += n
+        assert rel_err(outs[0], outs[1]) < TOL[dtype] / 3, (items[0], len(items))
+        return outs[0]
+
+    live = list(seqs)
+    for i in range(0, n_req, 8):                          # prompts of different lengths, a few a step
+        both([(r, 20 + (j * 7) % 40) for j, r in enumerate(live[i:i + 8])])
+    before = with_graphs.graphs.replays
+    for step in range(12):
+        both([(r, 1) for r in live])                      # one bucket, replayed
+        if step == 3:                                     # eager work between replays: a portion of a prompt
+            both([(live[0], 9)])
+        if step == 6:                                     # requests leave: a smaller batch, another bucket
+            for r in live[-2:]:
+                with_graphs.free_request(r)
+                eager.free_request(r)
+            live = live[:-2]
+    assert with_graphs.graphs.replays - before >= 12
+    # a longer context: the next bucket of the context length
+    both([(r, 240 if which == "B" else 120) for r in live[:3]])
+    for _ in range(3):
+        both([(r, 1) for r in live])
+    keys = set(with_graphs.graphs.steps)
+    assert len(keys) >= 2
+    if which == "B":                                      # 70 and 68 requests pad to 80 rows; 512 is the second context bucket
+        assert {(80, 256), (80, 512)} <= keys
