@@ -98,8 +98,11 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   }
   const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+  // Workgroups start their walk over K at different runs (and wrap round): if all walked in step, the
+  // rows read at one moment, a whole K apart from each other, would fall on few memory channels.
+  const int rot = (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)n_runs);
   auto gload = [&](GwRegs<MT, WV>& R, int run) {
-    const int k = run * GW_KS;
+    const int k = (run + rot < n_runs ? run + rot : run + rot - n_runs) * GW_KS;
     const bool wok = kb + k + lc * 8 < ke;       // K and the split are multiples of 8: a chunk is in or out
     const bool kok = kb + k + ac * 8 < ke;
 #pragma unroll
