@@ -14,7 +14,7 @@
 //
 // A workgroup owns 16*NT output features. Its waves split K: wave w takes the
 // k-runs w, w + WAVES, ... of U*32 elements, so together they walk each weight
-// row front to back. Loads for the next run are in flight while the current
+// row, from a start that differs from workgroup to workgroup, once round. Loads for the next run are in flight while the current
 // one is multiplied. The waves' partial sums are added through LDS in a fixed
 // order (deterministic; no atomics).
 //
@@ -116,9 +116,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       for (int i = 0; i < NI; ++i) ar[mt][i] = (ok && aok[mt][i]) ? *(const bf16x8_t*)(ap[mt][i] + k0) : zero;
   };
 
+  // A workgroup's waves walk K together, a span of WAVES runs a step. Workgroups start at different
+  // steps and wrap round: in step, the rows read at one moment (a whole K apart from each other, at
+  // the same offset) fall on few memory channels. A run past K loads nothing and multiplies zeros.
   const int span = WAVES * KS;
-  int k0 = wave * KS;
-  if (k0 < K) gload(k0);
+  const int n_steps = (K + span - 1) / span;
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)n_steps);
+  auto k_of = [&](int step) {
+    const int q = step + rot < n_steps ? step + rot : step + rot - n_steps;
+    return q * span + wave * KS;
+  };
+  gload(k_of(0));
   // This wave's share of the rows' partial sums, p = 4 wave + g, + 4 WAVES, ...: the first SS_HELD of a
   // lane are asked for here, behind the first weights, and not touched before the loop is over, so
   // that no wait for them holds up the weight stream; any further ones are read after the loop.
@@ -135,7 +143,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       }
     }
   }
-  for (; k0 < K; k0 += span) {
+  for (int step = 0; step < n_steps; ++step) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -149,7 +157,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     // the tile is the wave's own: its LDS operations complete in order, so waiting
     // for them is all the ordering the re-layout needs
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (k0 + span < K) gload(k0 + span);
+    if (step + 1 < n_steps) gload(k_of(step + 1));
     bf16x8_t a[NT][U], b[MT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
