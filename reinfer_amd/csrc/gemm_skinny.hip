@@ -121,7 +121,9 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   // the same offset) fall on few memory channels. A run past K loads nothing and multiplies zeros.
   const int span = WAVES * KS;
   const int n_steps = (K + span - 1) / span;
-  const int rot = (int)((blockIdx.x * 7u) % (unsigned)n_steps);
+  // (Measured: a gain where the grid is larger than the chip holds at once or K is long; a small loss
+  // at 6144 x 4096, where all workgroups run side by side and share the activations they read in step.)
+  const int rot = (gridDim.x > 512 || K > 8192) ? (int)((blockIdx.x * 7u) % (unsigned)n_steps) : 0;
   auto k_of = [&](int step) {
     const int q = step + rot < n_steps ? step + rot : step + rot - n_steps;
     return q * span + wave * KS;

@@ -1,4 +1,5 @@
-// Weight-streaming product for 17 to 64 rows:  C[M,N] = A[M,K] . W[N,K]^T, bfloat16 in, float
+// Weight-streaming product for up to 64 rows (the faster of the two from 17 rows on, and for wide gated
+// products below that):  C[M,N] = A[M,K] . W[N,K]^T, bfloat16 in, float
 // accumulation on the matrix cores.
 //
 // With more than one row tile the activations weigh as much as the weights: a workgroup that
@@ -144,6 +145,23 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
   for (int d = 0; d < GW_DEPTH; ++d)
     if (d < n_runs) gload(R[d], d);
+  // The carried norm's partial sums of row mt*16 + r, parts g, g + 4, ... a lane: the first GW_HELD of a
+  // lane are asked for here, behind the first weights, and not touched before the loop is over, so that
+  // no wait for them holds up the weight stream (a producer with 16 columns a workgroup leaves 256 of
+  // them for a width of 4096); any further ones are read after the loop.
+  constexpr int GW_HELD = MT == 1 ? 64 : (MT == 2 ? 16 : 4);
+  float held[MT][GW_HELD];
+  if (EPI != WEPI_PARTIAL && nf.in_ss) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+#pragma unroll
+      for (int j = 0; j < GW_HELD; ++j) {
+        const int p = g + 4 * j;
+        held[mt][j] = (m < M && p < nf.in_parts) ? nf.in_ss[(size_t)p * M + m] : 0.f;
+      }
+    }
+  }
   for (int run = 0; run < n_runs; run += GW_DEPTH) {  // n_runs is the same in every thread of the workgroup
 #pragma unroll
     for (int d = 0; d < GW_DEPTH; ++d)
@@ -154,8 +172,15 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
-    if (EPI != WEPI_PARTIAL && nf.in_ss && m < M) {      // a split product is scaled when its parts are added
-      const float rstd = gw_rstd(nf, m, M);
+    if (EPI != WEPI_PARTIAL && nf.in_ss) {               // a split product is scaled when its parts are added
+      float t = 0.f;                                     // a fixed order: a lane's parts ascending, then the lane groups
+#pragma unroll
+      for (int j = 0; j < GW_HELD; ++j) t += held[mt][j];
+      if (m < M)
+        for (int p = g + 4 * GW_HELD; p < nf.in_parts; p += 4) t += nf.in_ss[(size_t)p * M + m];
+      t += __shfl_xor(t, 16, RA_WAVE);
+      t += __shfl_xor(t, 32, RA_WAVE);
+      const float rstd = rsqrtf(t * nf.in_inv_width + nf.in_eps);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[mt][i] *= rstd;
     }
@@ -268,13 +293,16 @@ static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_
   if (partial) *partial = emits || *S > 1;
 }
 
-// 1 where this kernel beats ra_gemm_skinny (measured on MI355X at 24 to 64 rows): from 17 rows on,
+// 1 where this kernel beats ra_gemm_skinny (measured on MI355X at 4 to 64 rows): from 17 rows on,
 // except a small product whose K has to be cut (4096 x 4096: the second launch costs more than the
-// shared activations save).
+// shared activations save); below that for the gated product of a wide feed-forward.
 extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
-  if (M < 17 || M > 64) return 0;
+  if (M < 1 || M > 64) return 0;
   int waves, S, kps;
   gw_split(epilogue, N, K, &waves, &S, &kps);
+  // below 17 rows only the gated product of a wide feed-forward: one K range, enough workgroups to fill
+  // the chip (measured at 4 to 16 rows, 24576 x 4096: 37 us against 39 to 42)
+  if (M < 17) return (epilogue == WEPI_SILU_PAIRS && S == 1 && (N + waves * 16 - 1) / (waves * 16) >= 192) ? 1 : 0;
   return (S == 1 || (long)N * K > 4096L * 4096L) ? 1 : 0;
 }
 

@@ -421,7 +421,10 @@ class HipKernels:
         norm_args = (_ptr(ss), parts, float(eps or 0.0), int(width or 0), _ptr(w),
                      _tag(w, "norm weight") if w is not None else 0, _ptr(xo),
                      xo.stride(0) if xo is not None else 0, _ptr(so))
-        if M <= self.NORM_SKINNY_ROWS:
+        # the gated product of a wide feed-forward goes to the other kernel at every row count; it
+        # takes row sums (any number of parts) and never emits
+        gated_wide = epilogue == 1 and emit is None and bool(library.load().ra_gemm_wide_preferred(epilogue, M, N, K))
+        if M <= self.NORM_SKINNY_ROWS and not gated_wide:
             library.call("ra_gemm_skinny_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                          _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), *norm_args,
                          _stream())
