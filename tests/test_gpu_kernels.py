@@ -153,10 +153,10 @@ def rope_reference(x, positions, theta, rotary_dim, style):
 @pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [
     (4, 2, 16, 16, 0, True), (14, 2, 48, 48, 0, True), (5, 5, 128, 128, 0, True),
     (3, 1, 80, 32, 0, False), (6, 3, 64, 64, 1, True), (32, 8, 128, 128, 0, True), (2, 1, 256, 256, 0, True)])
-@pytest.mark.parametrize("T", [11, 45])       # few tokens: a wave per head; many: a workgroup per token
+@pytest.mark.parametrize("T", [11, 45, 200])  # few tokens: a wave per head; from 192: a workgroup per token
 def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm, T):
     torch.manual_seed(d + Hq)
-    bs, nblk, eps, theta = 16, 9, 1e-6, 10000.0
+    bs, nblk, eps, theta = 16, max(9, T // 16 + 3), 1e-6, 10000.0
     width = (Hq + 2 * Hkv) * d
     qkv = torch.randn(T, width, device=DEV).to(DT[dtype])
     src = qkv.clone()
