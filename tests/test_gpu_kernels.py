@@ -542,6 +542,38 @@ def test_rmsnorm_carried_by_two_products(M, N, K, wdt):
         close(out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
 
 
+@pytest.mark.parametrize("M", [3, 16])
+def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
+    """Up to 16 rows the product before the norm writes one partial sum per 16 columns (256 for a
+    width of 4096); a gated product wide enough to fill the chip goes to the kernel whose waves
+    share the activations at every row count, and adds them up itself."""
+    torch.manual_seed(M)
+    N, K, J, eps = 4096, 256, 9216, 1e-6
+    a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    stream = torch.randn(M, N, device=DEV) * 3
+    stream[M // 2] *= 30
+    nw = (1 + 0.3 * torch.randn(N, device=DEV)).to(torch.bfloat16)
+    parts = ops().skinny_row_parts(M, N)
+    assert parts == N // 16
+    xs = torch.empty((M, N), device=DEV, dtype=torch.bfloat16)
+    ss = torch.empty((parts, M), device=DEV)
+    ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss))
+    normed = stream.double() * torch.rsqrt((stream.double() ** 2).mean(1, keepdim=True) + eps) * nw.double()
+    wg = (torch.randn(J, N, device=DEV) * 2 / math.sqrt(N)).to(torch.bfloat16)
+    wu = (torch.randn(J, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
+    w = torch.stack([wg.view(J // 8, 8, N), wu.view(J // 8, 8, N)], dim=1).reshape(2 * J, N).contiguous()
+    assert kernels.library.load().ra_gemm_wide_preferred(1, M, 2 * J, N) == 1
+    out = torch.full((M, J), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().gated_linear(xs, w, out, row_sums=(ss, eps, N))
+    g, u = normed @ wg.double().T, normed @ wu.double().T
+    close(out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
+    plain_out = torch.full((M, J), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().gated_linear(xs, w, plain_out)                      # and without the carried norm
+    g, u = xs.double() @ wg.double().T, xs.double() @ wu.double().T
+    close(plain_out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
+
+
 def test_linear_dispatch_refuses_nothing_silently():
     """Sizes the MFMA kernel does not take go to the plain kernel, not to a wrong result."""
     x = torch.randn(5, 100, device=DEV).to(torch.bfloat16)[:, :99]       # K = 99, odd row stride
