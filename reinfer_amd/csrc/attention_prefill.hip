@@ -29,6 +29,7 @@
 // only the prompt itself, from position 0 (crates/cuda/src/fmha.rs:574-686;
 // crates/cuda/kernels/fmha_kernels.cu:96); this one is written here and reads
 // earlier context from the cache, so a prompt can be cut anywhere.
+#include <type_traits>
 #include "common.h"
 #include "reinfer_hip.h"
 
@@ -78,7 +79,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   const int kvh = blockIdx.y / n_hgrp, hgrp = blockIdx.y % n_hgrp;
   const int seq = tile_info[tile * 4 + 0];
   const int row0 = tile_info[tile * 4 + 1];
-  const int nq = tile_info[tile * 4 + 2];
+  // n queries in the low half; above it, optionally, which of a wave's NC column tiles this workgroup
+  // computes (bit j; 0 = all): a tile with many keys can be given to two workgroups, each with half of
+  // the heads, so that a launch of about as many tiles as the chip has CUs does not last as long as its
+  // heaviest tile while the CUs of the light ones idle.
+  const int nq_word = tile_info[tile * 4 + 2];
+  const int nq = nq_word & 0xffff;
+  const int col_bits = (nq_word >> 16) & ((1 << NC) - 1);
+  const int col_mask = col_bits ? col_bits : (1 << NC) - 1;
   const int pos0 = tile_info[tile * 4 + 3];
   const int* table = block_tables + (size_t)seq * max_blocks;
 
@@ -90,7 +98,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   for (int j = 0; j < NC; ++j) {
     const int c = wave * NC + j;
     qi[j] = (c / HG) * 16 + r;
-    q_live[j] = qi[j] < nq;
+    q_live[j] = qi[j] < nq && ((col_mask >> j) & 1);
     const int head = kvh * G + hgrp * HG + c % HG;
     const bf16_t* qp = q + (size_t)(row0 + (q_live[j] ? qi[j] : 0)) * q_stride + (size_t)head * d;
 #pragma unroll
@@ -214,24 +222,33 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         for (int ot = 0; ot < NOT; ++ot) va[ot] = v_operand(ot);
         __builtin_amdgcn_sched_barrier(0);     // the reads stay ahead of the products
       }
-      // scores S^T[key][column] for 2 sub-tiles of 16 keys
+      // scores S^T[key][column] for 2 sub-tiles of 16 keys, of the column tiles jlo .. jhi - 1
       f32x4_t s[2][NC];
+      auto scores = [&](auto jlo_c, auto jhi_c) {
+        constexpr int jlo = decltype(jlo_c)::value, jhi = decltype(jhi_c)::value;
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-        for (int j = 0; j < NC; ++j) s[ks][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+          for (int j = 0; j < NC; ++j) s[ks][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          if (dt * 32 < d) {
-            bf16x8_t a;
-            if constexpr (AHEAD) a = ka[ks][dt];
-            else a = k_operand(ks, dt);
+          for (int dt = 0; dt < NDT; ++dt) {
+            if (dt * 32 < d) {
+              bf16x8_t a;
+              if constexpr (AHEAD) a = ka[ks][dt];
+              else a = k_operand(ks, dt);
 #pragma unroll
-            for (int j = 0; j < NC; ++j)
-              s[ks][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j][dt], s[ks][j], 0, 0, 0);
+              for (int j = jlo; j < jhi; ++j)
+                s[ks][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j][dt], s[ks][j], 0, 0, 0);
+            }
           }
         }
-      }
+      };
+      using I0 = std::integral_constant<int, 0>;
+      using I1 = std::integral_constant<int, 1>;
+      using IN = std::integral_constant<int, NC>;
+      if (NC == 1 || col_mask == (1 << NC) - 1) scores(I0{}, IN{});
+      else if (col_mask == 1) scores(I0{}, I1{});
+      else scores(I1{}, IN{});
       // keys strictly inside every query's view need no mask
       const bool inner = kh + 31 <= w_first_pos && w_qend <= nq &&
                          (window <= 0 || kh >= w_last_pos - window + 1);
@@ -253,6 +270,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
       // matrix core works on them while the next tile's probabilities are computed.
 #pragma unroll
       for (int j = 0; j < NC; ++j) {
+        if (!((col_mask >> j) & 1)) continue;            // the other workgroup's column tile
         // Probabilities against the running maximum m first; m follows the true maximum only when
         // some probability comes out above 2^8 (the true maximum has grown by more than 8 in the
         // exponent): until then float sums and bfloat16 operands hold the larger values as well, and
@@ -371,6 +389,17 @@ extern "C" int ra_attention_prefill_supports(int Hq, int Hkv, int d, int block_s
 extern "C" int ra_attention_prefill_tile(int Hq, int Hkv, int d) {
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || d <= 0) return 64;
   return 16 * fp_shape(Hq, Hkv, d).runs;
+}
+
+// Column tiles a wave holds for these sizes (2: a tile's workgroup can be split in two by the high half of
+// the tile's query count, see the kernel) and workgroups a query tile makes (KV heads x head groups).
+extern "C" int ra_attention_prefill_columns(int Hq, int Hkv, int d) {
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || d <= 0) return 1;
+  return fp_shape(Hq, Hkv, d).nc;
+}
+extern "C" int ra_attention_prefill_groups(int Hq, int Hkv, int d) {
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || d <= 0) return 1;
+  return Hkv * ((Hq / Hkv) / fp_shape(Hq, Hkv, d).hg);
 }
 
 extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride,

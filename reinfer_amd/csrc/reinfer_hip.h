@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 11
+#define RA_ABI_VERSION 12
 
 #ifdef __cplusplus
 extern "C" {
@@ -90,9 +90,14 @@ int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, 
                         int chunk, int max_chunks, float* part_o, float* part_ml, hipStream_t stream);
 
 // bfloat16 flash prefill over query tiles; tile_info holds 4 ints per tile:
-// request row in block_tables, first token row, number of queries (<= tile), first position
+// request row in block_tables, first token row, number of queries (<= tile), first position.
+// Where ra_attention_prefill_columns() is 2, bits 16-17 of the third may name the half of the heads a
+// workgroup computes (1 or 2; 0 or 3: all): the same tile listed twice, once with each, is computed by
+// two workgroups. A tile makes ra_attention_prefill_groups() workgroups.
 int ra_attention_prefill_supports(int Hq, int Hkv, int d, int block_size);
 int ra_attention_prefill_tile(int Hq, int Hkv, int d);
+int ra_attention_prefill_columns(int Hq, int Hkv, int d);
+int ra_attention_prefill_groups(int Hq, int Hkv, int d);
 int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                          const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
                          int n_tiles, int block_size, int Hq, int Hkv, int d, float scale, int window,

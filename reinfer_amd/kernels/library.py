@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 
 class KernelLibraryError(RuntimeError):
@@ -71,8 +71,9 @@ def load() -> ctypes.CDLL:
             getattr(lib, name).argtypes = [c_int, c_int, c_int, c_int]
         lib.ra_attention_decode_slots.restype = c_int
         lib.ra_attention_decode_slots.argtypes = [c_int, c_int, c_int]
-        lib.ra_attention_prefill_tile.restype = c_int
-        lib.ra_attention_prefill_tile.argtypes = [c_int, c_int, c_int]
+        for name in ("ra_attention_prefill_tile", "ra_attention_prefill_columns", "ra_attention_prefill_groups"):
+            getattr(lib, name).restype = c_int
+            getattr(lib, name).argtypes = [c_int, c_int, c_int]
         lib.ra_gemm_skinny_max_rows.restype = c_int
         lib.ra_gemm_skinny_max_rows.argtypes = []
         lib.ra_gemm_skinny_row_parts.restype = c_int

@@ -674,6 +674,16 @@ def test_attention_prefill(Hq, Hkv, d):
                                     tiles, len(info) // 4)
             ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
             close(out, ref, 2 ** -7)
+            if kernels.library.load().ra_attention_prefill_columns(Hq, Hkv, d) == 2 and window != 100:
+                # every other tile given to two workgroups, each with one of a wave's two column tiles
+                cut = []
+                for k in range(len(info) // 4):
+                    i, row, n, pos = info[4 * k:4 * k + 4]
+                    cut += [i, row, n | (1 << 16), pos, i, row, n | (2 << 16), pos] if k % 2 == 0 else [i, row, n, pos]
+                out2 = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+                ops().attention_prefill(q.view(T, Hq * d), Hq * d, out2, kt(kc), vt(vc), batch, Hq, Hkv, d, scale,
+                                        window, 0, torch.tensor(cut, dtype=torch.int32, device=DEV), len(cut) // 4)
+                assert torch.equal(out2, out)             # the same arithmetic, column tile by column tile
 
 
 def test_attention_dispatch_mixed_batch():
@@ -687,8 +697,14 @@ def test_attention_dispatch_mixed_batch():
     out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
     ops().attention(q.view(T, -1), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, d ** -0.5, 0, 0)
     tile = kernels.library.load().ra_attention_prefill_tile(Hq, Hkv, d)
-    plan = batch.extra[("attention_plan", tile)]
-    assert plan["n_decode"] == 5 and plan["n_tiles"] == -(-70 // tile) + 1
+    (plan,) = [v for k, v in batch.extra.items() if isinstance(k, tuple) and k[:2] == ("attention_plan", tile)]
+    listed = plan["tiles"].view(-1, 4).tolist()
+    assert plan["n_decode"] == 5 and plan["n_tiles"] == len(listed)
+    rows = sorted({t[1] for t in listed})
+    assert len(rows) == -(-70 // tile) + 1                  # the query tiles themselves
+    for row in rows:                                        # each listed whole, or once for each half of the heads
+        marks = sorted(t[2] >> 16 for t in listed if t[1] == row)
+        assert marks in ([0], [1, 2])
     close(out, attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, d ** -0.5, 0), 2 ** -7)
 
 
