@@ -189,6 +189,20 @@ extern "C" int ra_add_rmsnorm(float* resid, const void* delta, const void* weigh
 #define QK_WAVES 4
 #define QK_MAX_D 512
 
+// The q/k/v product as the K ranges of a split product left it, not yet added (parts null: qkv holds the
+// finished product and q is rotated in place): float [n_ranges][T][width], added here in range order, with
+// the row factor of an RMSNorm carried by that product (in_ss null: none); the rotated q then goes to q_out.
+struct QkSums {
+  const float* parts;
+  int n_ranges;
+  size_t range_stride;     // T * width
+  const float* in_ss;      // [in_parts][T]
+  int in_parts;
+  float in_eps, in_inv_width;
+  void* q_out;             // [T][q_stride] in the activations' type
+  int q_stride;
+};
+
 template <typename TA, typename TW>
 __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w,
                                           const TW* __restrict__ k_w, float eps,
@@ -196,7 +210,7 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
                                           const float* __restrict__ inv_freq, int rotary_dim,
                                           int rope_style, const int* __restrict__ slots,
                                           TA* __restrict__ kcache, TA* __restrict__ vcache,
-                                          int block_size, int Hq, int Hkv, int d) {
+                                          int block_size, int Hq, int Hkv, int d, QkSums sm) {
   __shared__ float buf[QK_WAVES][QK_MAX_D];
   const int lane = threadIdx.x & (RA_WAVE - 1);
   const int wave = threadIdx.x / RA_WAVE;
@@ -219,10 +233,27 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   float* b = buf[wave];
   float ss = 0.f;
   if (live) {
-    for (int i = lane; i < d; i += RA_WAVE) {
-      float v = to_f32(u[i]);
-      b[i] = v;
-      ss += v * v;
+    if (sm.parts) {
+      float row = 1.f;
+      if (sm.in_ss) {
+        float tsum = 0.f;
+        for (int p = 0; p < sm.in_parts; ++p) tsum += sm.in_ss[(size_t)p * gridDim.y + t];      // fixed order
+        row = rsqrtf(tsum * sm.in_inv_width + sm.in_eps);
+      }
+      const float* src = sm.parts + ((size_t)t * n_heads + head) * d;
+      for (int i = lane; i < d; i += RA_WAVE) {
+        float v = 0.f;
+        for (int r = 0; r < sm.n_ranges; ++r) v += src[(size_t)r * sm.range_stride + i];        // range order
+        v *= row;
+        b[i] = v;
+        ss += v * v;
+      }
+    } else {
+      for (int i = lane; i < d; i += RA_WAVE) {
+        float v = to_f32(u[i]);
+        b[i] = v;
+        ss += v * v;
+      }
     }
   }
   __syncthreads();
@@ -240,8 +271,9 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   }
   if (!is_q && !slab) return;
   // where element i of the head goes: in place for q, the cache slab for k
+  TA* q_to = sm.parts ? (TA*)sm.q_out + (size_t)t * sm.q_stride + (size_t)head * d : u;
   auto put = [&](int i, float v) {
-    if (is_q) u[i] = from_f32<TA>(v);
+    if (is_q) q_to[i] = from_f32<TA>(v);
     else slab[cache_k_index(off, i, d)] = from_f32<TA>(v);
   };
   const float pos = (float)positions[t];
@@ -331,11 +363,11 @@ qk_norm_rope_cache_token_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w
   }
 }
 
-extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
-                                     int weight_dtype, float eps, const int* positions,
-                                     const float* inv_freq, int rotary_dim, int rope_style,
-                                     const int* slots, void* kcache, void* vcache, int block_size,
-                                     int n_tokens, int Hq, int Hkv, int d, hipStream_t stream) {
+static int qk_norm_rope_cache_impl(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
+                                   int weight_dtype, float eps, const int* positions,
+                                   const float* inv_freq, int rotary_dim, int rope_style,
+                                   const int* slots, void* kcache, void* vcache, int block_size,
+                                   int n_tokens, int Hq, int Hkv, int d, const QkSums& sm, hipStream_t stream) {
   RA_CHECK(n_tokens > 0, "qk_norm_rope_cache: no tokens");
   RA_CHECK(Hq > 0 && Hkv > 0 && d > 0, "qk_norm_rope_cache: bad head sizes (%d, %d, %d)", Hq, Hkv, d);
   RA_CHECK(d <= QK_MAX_D, "qk_norm_rope_cache: head size %d above the supported %d", d, QK_MAX_D);
@@ -351,7 +383,7 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
   // with few tokens (decode) a wave per head spreads over more of the chip (measured at 32 heads of 128:
   // 3.2 against 4.4 us at 64 tokens, 3.9 against 4.7 at 128, 6.2 against 5.4 at 255)
   const bool pow2 = (d & (d - 1)) == 0 && d >= 16 && d <= 256;
-  if (pow2 && n_tokens >= 192 && rope_style == 0 && rotary_dim == d && ((uintptr_t)qkv % 16) == 0 &&
+  if (!sm.parts && pow2 && n_tokens >= 192 && rope_style == 0 && rotary_dim == d && ((uintptr_t)qkv % 16) == 0 &&
       (q_weight == nullptr || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0))) {
 #define RA_TOK2(TA, TW, LPH)                                                                              \
   qk_norm_rope_cache_token_kernel<TA, TW, LPH><<<n_tokens, 256, 0, stream>>>(                             \
@@ -378,7 +410,7 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
 #define RA_GO(TA, TW)                                                                              \
   qk_norm_rope_cache_kernel<TA, TW><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(                      \
       (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, rotary_dim,   \
-      rope_style, slots, (TA*)kcache, (TA*)vcache, block_size, Hq, Hkv, d)
+      rope_style, slots, (TA*)kcache, (TA*)vcache, block_size, Hq, Hkv, d, sm)
   if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_GO(float, float);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_GO(bf16_t, bf16_t);
   else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_GO(bf16_t, float);
@@ -386,6 +418,48 @@ extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_wei
 #undef RA_GO
   RA_LAUNCH_CHECK("qk_norm_rope_cache");
   return 0;
+}
+
+extern "C" int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
+                                     int weight_dtype, float eps, const int* positions,
+                                     const float* inv_freq, int rotary_dim, int rope_style,
+                                     const int* slots, void* kcache, void* vcache, int block_size,
+                                     int n_tokens, int Hq, int Hkv, int d, hipStream_t stream) {
+  RA_CHECK(qkv != nullptr, "qk_norm_rope_cache: no q/k/v rows");
+  const QkSums none = {};
+  return qk_norm_rope_cache_impl(qkv, act_dtype, q_weight, k_weight, weight_dtype, eps, positions, inv_freq,
+                                 rotary_dim, rope_style, slots, kcache, vcache, block_size, n_tokens, Hq, Hkv, d,
+                                 none, stream);
+}
+
+// The same from the float partial results of a product cut into K ranges ([n_ranges][n_tokens][width],
+// width = (Hq + 2 Hkv) d), which are added here, in range order, instead of by a kernel of their own; with
+// in_ss ([in_parts][n_tokens] partial sums of squares, eps, width) the rows are also scaled by the RMSNorm
+// that product carried. The rotated q goes to q_out ([n_tokens][q_stride], the cache's type).
+extern "C" int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, const float* in_ss, int in_parts,
+                                          float in_eps, int in_width, void* q_out, int q_stride, int act_dtype,
+                                          const void* q_weight, const void* k_weight, int weight_dtype,
+                                          float eps, const int* positions, const float* inv_freq,
+                                          int rotary_dim, int rope_style, const int* slots, void* kcache,
+                                          void* vcache, int block_size, int n_tokens, int Hq, int Hkv, int d,
+                                          hipStream_t stream) {
+  RA_CHECK(parts && n_ranges >= 1 && q_out, "qk_norm_rope_cache_sums: partial results and a place for q are needed");
+  RA_CHECK(q_stride >= Hq * d, "qk_norm_rope_cache_sums: q rows of %d elements do not hold %d heads of %d", q_stride, Hq, d);
+  RA_CHECK(in_ss == nullptr || (in_parts > 0 && in_width > 0 && in_eps >= 0.f),
+           "qk_norm_rope_cache_sums: row sums need parts (%d), width (%d) and eps", in_parts, in_width);
+  QkSums sm = {};
+  sm.parts = parts;
+  sm.n_ranges = n_ranges;
+  sm.range_stride = (size_t)n_tokens * (size_t)(Hq + 2 * Hkv) * (size_t)d;
+  sm.in_ss = in_ss;
+  sm.in_parts = in_parts;
+  sm.in_eps = in_eps;
+  sm.in_inv_width = in_ss ? 1.f / (float)in_width : 0.f;
+  sm.q_out = q_out;
+  sm.q_stride = q_stride;
+  return qk_norm_rope_cache_impl(nullptr, act_dtype, q_weight, k_weight, weight_dtype, eps, positions, inv_freq,
+                                 rotary_dim, rope_style, slots, kcache, vcache, block_size, n_tokens, Hq, Hkv, d,
+                                 sm, stream);
 }
 
 // ---------------------------------------------------------------------------

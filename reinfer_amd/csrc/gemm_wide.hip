@@ -406,6 +406,48 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
 #undef RA_GWL
 }
 
+// K ranges that ra_gemm_wide_partial cuts [M, N, K] into (its result has that many [M, N] float planes).
+extern "C" int ra_gemm_wide_ranges(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int waves, S, kps;
+  bool partial;
+  gw_split(WEPI_PLAIN, N, K, &waves, &S, &kps, &partial, true);
+  return S;
+}
+
+// Only the first half of a split product: P[s][m][n] = A[m, range s] . W[n, range s]^T, float, for a
+// consumer that adds the ranges itself (in range order) instead of the adding kernel.
+extern "C" int ra_gemm_wide_partial(const void* A, const void* W, float* P, long p_floats, int M, int N, int K,
+                                    int lda, hipStream_t stream) {
+  RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
+  RA_CHECK(M <= 64, "gemm_wide: %d rows; this kernel takes at most 64", M);
+  RA_CHECK(K % 8 == 0 && lda % 8 == 0 && lda >= K, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
+  RA_CHECK(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)P % 16) == 0,
+           "gemm_wide: operands must be 16-byte aligned");
+  int waves, S, kps;
+  bool partial;
+  gw_split(WEPI_PLAIN, N, K, &waves, &S, &kps, &partial, true);
+  RA_CHECK(P && p_floats >= (long)S * M * N, "gemm_wide: %d ranges of [%d, %d] need %ld floats, got %ld", S, M, N,
+           (long)S * M * N, p_floats);
+  const WideNorm nf = {};
+#define RA_GWP(MT, WV)                                                                                  \
+  gemm_wide_kernel<MT, WV, WEPI_PARTIAL, float><<<dim3((N + WV * 16 - 1) / (WV * 16), S), WV * RA_WAVE, 0, stream>>>( \
+      (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, P, N, M, N, K, kps, nf)
+#define RA_GWPM(MT)              \
+  do {                           \
+    if (waves == 6) RA_GWP(MT, 6); \
+    else RA_GWP(MT, 8);          \
+  } while (0)
+  if (M <= 16) RA_GWPM(1);
+  else if (M <= 32) RA_GWPM(2);
+  else if (M <= 48) RA_GWPM(3);
+  else RA_GWPM(4);
+#undef RA_GWPM
+#undef RA_GWP
+  RA_LAUNCH_CHECK("gemm_wide partial");
+  return 0;
+}
+
 extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                             int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                             hipStream_t stream) {

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 12
+#define RA_ABI_VERSION 13
 
 #ifdef __cplusplus
 extern "C" {
@@ -24,6 +24,14 @@ int ra_qk_norm_rope_cache(void* qkv, int act_dtype, const void* q_weight, const 
                           int weight_dtype, float eps, const int* positions, const float* inv_freq,
                           int rotary_dim, int rope_style, const int* slots, void* kcache, void* vcache,
                           int block_size, int n_tokens, int Hq, int Hkv, int d, hipStream_t stream);
+// The same from the partial results of ra_gemm_wide_partial (added here, in range order), optionally scaled
+// by the RMSNorm that product carried (in_ss [in_parts][n_tokens], eps, width); the rotated q goes to q_out.
+int ra_qk_norm_rope_cache_sums(const float* parts, int n_ranges, const float* in_ss, int in_parts, float in_eps,
+                               int in_width, void* q_out, int q_stride, int act_dtype, const void* q_weight,
+                               const void* k_weight, int weight_dtype, float eps, const int* positions,
+                               const float* inv_freq, int rotary_dim, int rope_style, const int* slots,
+                               void* kcache, void* vcache, int block_size, int n_tokens, int Hq, int Hkv, int d,
+                               hipStream_t stream);
 
 // gate_up is [T, 2I]: group == 0: gate columns [0, I), up columns [I, 2I); group > 0: gate and
 // up interleaved in runs of `group` columns (gate run, then the up run of the same features)
@@ -60,6 +68,9 @@ int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* 
 // workgroup's waves; ra_gemm_wide_preferred says where it is the faster of the two (17 rows and
 // more, not the smallest products). Small N cuts K into ranges whose float partial results need
 // `ra_gemm_wide_scratch(...)` floats of scratch (0: none needed).
+int ra_gemm_wide_ranges(int M, int N, int K);          // K ranges of ra_gemm_wide_partial's result
+int ra_gemm_wide_partial(const void* A, const void* W, float* P, long p_floats, int M, int N, int K, int lda,
+                         hipStream_t stream);         // P[range][m][n] float, for a consumer that adds the ranges
 int ra_gemm_wide_preferred(int epilogue, int M, int N, int K);
 long ra_gemm_wide_scratch(int epilogue, int M, int N, int K, int emits);
 int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 
 class KernelLibraryError(RuntimeError):
@@ -32,6 +32,8 @@ _SIGNATURES = {
     "ra_embed": [P, I, P, P, I, I, P],
     "ra_add_rmsnorm": [P, P, P, I, P, I, P, I, I, F, P],
     "ra_qk_norm_rope_cache": [P, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
+    "ra_qk_norm_rope_cache_sums": [P, I, P, I, F, I, P, I, I, P, P, I, F, P, P, I, I, P, P, P, I, I, I, I, I, P],
+    "ra_gemm_wide_partial": [P, P, P, c_long, I, I, I, I, P],
     "ra_silu_mul": [P, P, I, I, I, I, P],
     "ra_attention_plain": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P, P],
@@ -82,6 +84,8 @@ def load() -> ctypes.CDLL:
         lib.ra_gemm_wide_scratch.argtypes = [c_int, c_int, c_int, c_int, c_int]
         lib.ra_gemm_wide_row_parts.restype = c_int
         lib.ra_gemm_wide_row_parts.argtypes = [c_int]
+        lib.ra_gemm_wide_ranges.restype = c_int
+        lib.ra_gemm_wide_ranges.argtypes = [c_int, c_int, c_int]
         lib.ra_gemm_wide_preferred.restype = c_int
         lib.ra_gemm_wide_preferred.argtypes = [c_int, c_int, c_int, c_int]
         if lib.ra_abi_version() != ABI_VERSION:

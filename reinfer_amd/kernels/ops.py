@@ -119,6 +119,69 @@ class HipKernels:
                      int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(),
                      vcache.data_ptr(), kcache.shape[2] * 16, T, num_heads, num_kv_heads, head_dim, _stream())
 
+    # ---- the q/k/v product left in K ranges for the kernel that consumes it
+    def linear_ranges(self, x: torch.Tensor, weight: torch.Tensor):
+        """x . weight^T as the float results of the K ranges it was cut into, [ranges, M, N], not yet
+        added, or None where that does not pay: only the products the split kernel takes (bfloat16,
+        17 to 64 rows) and cuts (few output features), whose adding kernel a consumer can save by
+        adding the ranges itself (``qk_norm_rope_cache(..., ranges=)``)."""
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2):
+            return None
+        M, K = x.shape
+        N = weight.shape[0]
+        if not (self.NORM_SKINNY_ROWS < M <= 64) or K % 8 or x.stride(1) != 1 or x.stride(0) % 8 \
+                or weight.shape != (N, K) or not weight.is_contiguous():
+            return None
+        lib = library.load()
+        S = int(lib.ra_gemm_wide_ranges(M, N, K))
+        if S < 2 or not lib.ra_gemm_wide_preferred(0, M, N, K):
+            return None
+        parts = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
+        library.call("ra_gemm_wide_partial", x.data_ptr(), weight.data_ptr(), parts.data_ptr(), parts.numel(),
+                     M, N, K, x.stride(0), _stream())
+        return parts
+
+    def qk_norm_rope_cache_ranges(self, ranges: torch.Tensor, row_sums, q_out: torch.Tensor,
+                                  q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                                  positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int,
+                                  rope_style: int, slots: torch.Tensor, kcache: torch.Tensor,
+                                  vcache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+        """``qk_norm_rope_cache`` on the result of ``linear_ranges``: the ranges are added here (in
+        range order), the rows scaled by the RMSNorm that the product carried (``row_sums`` = (ss
+        [parts, T], eps, width) or None), q normalised and rotated into ``q_out`` [T, heads * head_dim]."""
+        _dev(ranges, q_weight, k_weight, positions, inv_freq, slots, kcache, vcache, q_out)
+        S, T, width = ranges.shape
+        if width != (num_heads + 2 * num_kv_heads) * head_dim or ranges.dtype != torch.float32 \
+                or not ranges.is_contiguous():
+            raise ValueError(f"qk_norm_rope_cache: ranges {tuple(ranges.shape)} {ranges.dtype}, expected float32 "
+                             f"[ranges, T, {(num_heads + 2 * num_kv_heads) * head_dim}]")
+        self._check_cache("qk_norm_rope_cache", kcache, vcache, num_kv_heads, head_dim)
+        if q_out.dtype != kcache.dtype or q_out.shape != (T, num_heads * head_dim) or q_out.stride(1) != 1:
+            raise ValueError("qk_norm_rope_cache: q_out is [T, heads * head_dim] in the cache's dtype")
+        _int32(positions, "positions", T)
+        _int32(slots, "cache slots", T)
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() < rotary_dim // 2:
+            raise ValueError("qk_norm_rope_cache: inv_freq is float32 with rotary_dim/2 entries")
+        wtag = 0
+        for w in (q_weight, k_weight):
+            if w is not None:
+                if w.shape != (head_dim,):
+                    raise ValueError(f"qk_norm_rope_cache: head-norm weight {tuple(w.shape)}, expected [{head_dim}]")
+                wtag = _tag(w, "head-norm weight")
+        ss = None
+        parts, in_eps, in_width = 0, 0.0, 0
+        if row_sums is not None:
+            ss, in_eps, in_width = row_sums
+            _dev(ss)
+            if ss.dtype != torch.float32 or ss.dim() != 2 or ss.shape[1] != T or not ss.is_contiguous():
+                raise ValueError(f"qk_norm_rope_cache: row sums {tuple(ss.shape)} {ss.dtype}, expected float32 [parts, {T}]")
+            parts = ss.shape[0]
+        library.call("ra_qk_norm_rope_cache_sums", ranges.data_ptr(), S, _ptr(ss), parts, float(in_eps),
+                     int(in_width), q_out.data_ptr(), q_out.stride(0), _tag(q_out, "q"), _ptr(q_weight),
+                     _ptr(k_weight), wtag, float(eps), positions.data_ptr(), inv_freq.data_ptr(),
+                     int(rotary_dim), int(rope_style), slots.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
+                     kcache.shape[2] * 16, T, num_heads, num_kv_heads, head_dim, _stream())
+
     def silu_mul(self, gate_up: torch.Tensor, out: torch.Tensor, group: int = 0) -> None:
         """out = silu(gate) * up. ``group`` 0: gate_up is [gate | up]; ``group`` g > 0: runs of g
         gate columns and g up columns alternate."""

@@ -78,17 +78,29 @@ class GroupedQueryAttention:
         ops = kernels.current()
         x, row_sums = split_input(x)
         T = x.shape[0]
-        qkv = torch.empty((T, self.qkv_width), dtype=self.dtype, device=x.device)
-        if row_sums is None:
-            ops.linear(x, self.w_qkv, qkv, self.b_qkv)
-        else:
-            ops.linear_skinny(x, self.w_qkv, qkv, self.b_qkv, row_sums=row_sums)
         slots = batch.slots[cache.group] if cache.writes else batch.no_slots
-        ops.qk_norm_rope_cache(qkv, self.q_norm, self.k_norm, self.eps, batch.positions,
-                               self.position.inv_freq, self.position.rotary_dim, self.position.style,
-                               slots, cache.k, cache.v, self.num_heads, self.num_kv_heads, self.head_dim)
+        # a product that the kernels cut into K ranges may hand them over unadded: the kernel behind it
+        # adds them as it reads, which saves the adding kernel (and applies a carried norm's row factor)
+        in_ranges = getattr(ops, "linear_ranges", None)
+        ranges = in_ranges(x, self.w_qkv) if in_ranges is not None and self.b_qkv is None else None
+        if ranges is not None:
+            q_rows, q_stride = torch.empty((T, self.num_heads * self.head_dim), dtype=self.dtype, device=x.device), \
+                self.num_heads * self.head_dim
+            ops.qk_norm_rope_cache_ranges(ranges, row_sums, q_rows, self.q_norm, self.k_norm, self.eps,
+                                          batch.positions, self.position.inv_freq, self.position.rotary_dim,
+                                          self.position.style, slots, cache.k, cache.v, self.num_heads,
+                                          self.num_kv_heads, self.head_dim)
+        else:
+            q_rows, q_stride = torch.empty((T, self.qkv_width), dtype=self.dtype, device=x.device), self.qkv_width
+            if row_sums is None:
+                ops.linear(x, self.w_qkv, q_rows, self.b_qkv)
+            else:
+                ops.linear_skinny(x, self.w_qkv, q_rows, self.b_qkv, row_sums=row_sums)
+            ops.qk_norm_rope_cache(q_rows, self.q_norm, self.k_norm, self.eps, batch.positions,
+                                   self.position.inv_freq, self.position.rotary_dim, self.position.style,
+                                   slots, cache.k, cache.v, self.num_heads, self.num_kv_heads, self.head_dim)
         attn = torch.empty((T, self.num_heads * self.head_dim), dtype=self.dtype, device=x.device)
-        ops.attention(qkv, self.qkv_width, attn, cache.k, cache.v, batch, self.num_heads,
+        ops.attention(q_rows, q_stride, attn, cache.k, cache.v, batch, self.num_heads,
                       self.num_kv_heads, self.head_dim, self.scale, self.window, cache.group)
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(attn, self.w_o):

@@ -203,6 +203,56 @@ def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm, T):
     assert torch.isnan(vc.float().cpu().permute(0, 2, 1, 3)[untouched]).all()
 
 
+@pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [(4, 2, 16, 16, 0, True), (3, 1, 80, 32, 0, False),
+                                                      (6, 3, 64, 64, 1, True), (32, 8, 128, 128, 0, True)])
+@pytest.mark.parametrize("T,S,carried", [(5, 1, False), (33, 4, True), (64, 3, True), (20, 2, False)])
+def test_qk_norm_rope_cache_from_the_ranges_of_a_split_product(Hq, Hkv, d, rot, style, norm, T, S, carried):
+    """The same kernel fed with the float results of the K ranges of a split product, which it adds
+    itself, and with the partial sums of squares of an RMSNorm carried by that product: equal to
+    the plain kernel on the sum, scaled."""
+    torch.manual_seed(d + Hq + T)
+    bs, nblk, eps, theta = 16, T // 16 + 3, 1e-6, 10000.0
+    width = (Hq + 2 * Hkv) * d
+    ranges = torch.randn(S, T, width, device=DEV)
+    total = ranges.double().sum(0)
+    row_sums = None
+    if carried:
+        parts, hidden, neps = 3, 100, 1e-5
+        ss = torch.rand(parts, T, device=DEV) * hidden
+        row_sums = (ss, neps, hidden)
+        total = total * torch.rsqrt(ss.double().sum(0) / hidden + neps)[:, None]
+    qw = (torch.rand(d, device=DEV) + 0.5).to(torch.bfloat16) if norm else None
+    kw = (torch.rand(d, device=DEV) + 0.5).to(torch.bfloat16) if norm else None
+    g = torch.Generator().manual_seed(T)
+    positions = torch.randint(0, 128, (T,), generator=g).to(torch.int32).to(DEV)
+    slots_l = torch.randperm(nblk * bs, generator=g)[:T].tolist()
+    slots_l[T // 2] = -1
+    slots = torch.tensor(slots_l, dtype=torch.int32, device=DEV)
+    kc = torch.full((nblk, Hkv, bs // 16, 16 * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    vc = torch.full_like(kc, float("nan"))
+    j = torch.arange(max(rot // 2, 1), dtype=torch.float64)
+    inv_freq = (theta ** (-2.0 * j / max(rot, 1))).float().to(DEV)
+    q_out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().qk_norm_rope_cache_ranges(ranges, row_sums, q_out, qw, kw, eps, positions, inv_freq, rot, style, slots,
+                                    kc, vc, Hq, Hkv, d)
+    u = total.cpu().view(T, Hq + 2 * Hkv, d)
+    q, k, v = u[:, :Hq], u[:, Hq:Hq + Hkv], u[:, Hq + Hkv:]
+    if norm:
+        q = plain.head_norm(q, qw.double().cpu(), eps)
+        k = plain.head_norm(k, kw.double().cpu(), eps)
+    q_ref = rope_reference(q, positions.cpu(), theta, rot, style)
+    k_ref = rope_reference(k, positions.cpu(), theta, rot, style)
+    tol = OUT_TOL["bfloat16"]
+    kc, vc = unpack_k(kc, d), unpack_v(vc, d)
+    close(q_out.view(T, Hq, d), q_ref, tol)
+    for t, sl in enumerate(slots_l):
+        if sl < 0:
+            continue
+        close(kc[sl // bs, :, sl % bs, :], k_ref[t], tol)
+        close(vc[sl // bs, :, sl % bs, :], v[t], tol)
+    assert int(torch.isnan(kc.float()).any(-1).sum()) == (nblk * bs - (T - 1)) * Hkv
+
+
 def test_rotation_depends_on_distance_only():
     """<R_p q, R_t k> is a function of p - t: shift all positions and nothing changes."""
     Hq, Hkv, d, bs = 2, 1, 32, 16
