@@ -75,8 +75,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   const int r = lane & 15, g = lane >> 4;
   const int G = Hq / Hkv;
   const int n_hgrp = G / HG;
-  const int tile = gridDim.x - 1 - blockIdx.x;          // later tiles see more keys: start them first
-  const int kvh = blockIdx.y / n_hgrp, hgrp = blockIdx.y % n_hgrp;
+  // Workgroups go round the chip's XCDs, each with an L2 of its own, in the order of their numbers: the
+  // (KV head, head group) is the fast index, so that with 8 of them all query tiles of one KV head run on
+  // one XCD and its keys and values fill one L2 instead of all of them. Later tiles see more keys: they
+  // start first.
+  const int gy = Hkv * n_hgrp;
+  const int by = blockIdx.x % gy;
+  const int tile = gridDim.x / gy - 1 - blockIdx.x / gy;
+  const int kvh = by / n_hgrp, hgrp = by % n_hgrp;
   const int seq = tile_info[tile * 4 + 0];
   const int row0 = tile_info[tile * 4 + 1];
   // n queries in the low half; above it, optionally, which of a wave's NC column tiles this workgroup
@@ -418,7 +424,8 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
   const int G = Hq / Hkv;
   const int gy = Hkv * (G / sh.hg);
   RA_CHECK(gy <= 65535, "attention_prefill: too many heads for one launch");
-  dim3 grid(n_tiles, gy);
+  RA_CHECK((long)n_tiles * gy <= 0x7fffffffL, "attention_prefill: too many workgroups");
+  dim3 grid(n_tiles * gy);
   const float scale_log2 = scale * 1.4426950408889634f;
 #define RA_FP_GO(DM, NCC, EX)                                                                         \
   flash_prefill_kernel<DM, NCC, EX><<<grid, FP_THREADS, 0, stream>>>(                                 \
