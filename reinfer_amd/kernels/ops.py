@@ -272,6 +272,11 @@ class HipKernels:
                     tiles.extend((i, t + q0, min(tile, ql - q0), st + q0))
             t += ql
         n_tiles = len(tiles) // 4
+        if n_tiles > 1:
+            # the kernel starts the last listed tile first: list the tiles by the keys they see, so that
+            # the longest of every request start first, whatever the order of the requests
+            quads = sorted((tuple(tiles[4 * k:4 * k + 4]) for k in range(n_tiles)), key=lambda t: t[3] + t[2])
+            tiles = [v for t in quads for v in t]
         if 0 < n_tiles < room:
             by_keys = sorted(range(n_tiles), key=lambda k: -(tiles[4 * k + 3] + tiles[4 * k + 2]))
             twice = set(by_keys[:room - n_tiles])
