@@ -12,6 +12,7 @@ JSON line goes to standard output: ``value`` is decoded tokens a second at batch
 8; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the
 decode step against 8 TB/s by the bytes it must read (every weight once and the
 keys and values of the live requests); ``points`` holds batch 1 and batch 64.
+``--shape 4b`` and ``--shape 32b`` run the same measurement at the Qwen3-4B and Qwen3-32B layer sizes.
 The reference publishes no number at this size (its own are Qwen3-0.6B on a
 laptop GPU, bench/gate-fixture.md:66-74), so ``vs_baseline`` is null.
 """
@@ -37,6 +38,14 @@ QWEN3_8B = {
     "intermediate_size": 12288, "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
     "tie_word_embeddings": False, "max_position_embeddings": 4096, "attention_bias": False,
 }
+
+
+# the other two full-size shapes the engine is sized for (tied head at 2560 wide; 64 query heads at 5120 wide)
+QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, tie_word_embeddings=True,
+                max_position_embeddings=8192)
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64,
+                 intermediate_size=25600, max_position_embeddings=16384)
+SHAPES = {"8b": ("Qwen3-8B", QWEN3_8B), "4b": ("Qwen3-4B", QWEN3_4B), "32b": ("Qwen3-32B", QWEN3_32B)}
 
 
 def log(msg: str) -> None:
@@ -119,6 +128,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -133,7 +143,8 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
     kernels.current()
-    raw = dict(QWEN3_8B)
+    shape_name, shape = SHAPES[args.shape]
+    raw = dict(shape)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -144,7 +155,7 @@ def main() -> int:
     # a request decodes while later prompts are still being prefilled: one step a prompt
     blocks_per_req = -(-(args.prompt_len + max_batch + args.warmup + args.steps + 16) // block)
     num_blocks = max_batch * blocks_per_req + 8
-    log(f"building {raw['num_hidden_layers']} layers of the Qwen3-8B shape in {args.dtype}, random weights ...")
+    log(f"building {raw['num_hidden_layers']} layers of the {shape_name} shape in {args.dtype}, random weights ...")
     t0 = time.perf_counter()
     engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=block, num_blocks=num_blocks,
                        max_num_seqs=max_batch, max_num_batched_tokens=max(2048, args.prefill_tokens),
@@ -183,12 +194,12 @@ def main() -> int:
             log(f"decode batch {b}: {pms:.3f} ms a step, {points[f'decode_b{b}']:.0f} tok/s")
 
     out = {
-        "metric": "decode tok/s at batch 8 (Qwen3-8B shape, bf16, 2048-token prompts)",
+        "metric": f"decode tok/s at batch {args.batch} ({shape_name} shape, {dkey}, {args.prompt_len}-token prompts)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dkey, "data": "synthetic (uniform-random token ids, random weights N(0, 0.02))",
         "config": {
-            "model": "Qwen3-8B shape", "layers": raw["num_hidden_layers"], "layers_of_model": full_layers,
+            "model": f"{shape_name} shape", "layers": raw["num_hidden_layers"], "layers_of_model": full_layers,
             "hidden": raw["hidden_size"], "q_heads": raw["num_attention_heads"],
             "kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
             "intermediate": raw["intermediate_size"], "vocab": raw["vocab_size"],
