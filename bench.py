@@ -12,6 +12,8 @@ JSON line goes to standard output: ``value`` is decoded tokens a second at batch
 8; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the
 decode step against 8 TB/s by the bytes it must read (every weight once and the
 keys and values of the live requests); ``points`` holds batch 1 and batch 64.
+``--serve N`` runs a continuous-batching workload of N requests instead (the reference's replay harness
+feeds its scheduler synthetic arrivals the same way, crates/scheduler/src/replay.rs:180-217).
 ``--shape 4b`` and ``--shape 32b`` run the same measurement at the Qwen3-4B and Qwen3-32B layer sizes.
 The reference publishes no number at this size (its own are Qwen3-0.6B on a
 laptop GPU, bench/gate-fixture.md:66-74), so ``vs_baseline`` is null.
@@ -116,6 +118,56 @@ def prefill_run(engine, raw, tokens: int, reps: int, seed: int) -> float:
     return statistics.median(times)
 
 
+def serve_run(args, raw, shape_name: str) -> int:
+    """Continuous batching: ``args.serve`` requests arrive at once, prompts uniform in [64, 4096] tokens and
+    outputs uniform in [32, 512], prompts cut into portions under a 2,048-token step budget beside the
+    decoding requests. One JSON line: generated and total tokens a second over the whole run."""
+    import random
+    import torch
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.engine import LLMEngine
+    from reinfer_amd.sampling import SamplingParams
+    rng = random.Random(args.seed)
+    reqs = [(rng.randint(64, 4096), rng.randint(32, 512)) for _ in range(args.serve)]
+    raw["max_position_embeddings"] = max(raw["max_position_embeddings"], 4096 + 512 + 1)
+    block = 16
+    num_blocks = args.num_blocks or sum((p + o + block - 1) // block + 1 for p, o in reqs)
+    max_seqs = min(args.serve, 128)
+    log(f"building {raw['num_hidden_layers']} layers of the {shape_name} shape in {args.dtype}, {num_blocks} cache blocks ...")
+    engine = LLMEngine(config=config_from_dict(raw), seed=args.seed, dtype=args.dtype, block_size=block,
+                       num_blocks=num_blocks, max_num_seqs=max_seqs, max_num_batched_tokens=2048,
+                       max_model_len=raw["max_position_embeddings"])
+    g = torch.Generator().manual_seed(args.seed + 1)
+    for p, o in reqs:
+        engine.add_request(torch.randint(0, raw["vocab_size"], (p,), generator=g).tolist(),
+                           SamplingParams(temperature=0.0, max_tokens=o, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while engine.has_unfinished():
+        engine.step()
+        steps += 1
+        if steps % 200 == 0:
+            log(f"step {steps}: {len(engine.scheduler.running)} running, {len(engine.scheduler.waiting)} waiting")
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    t_in, t_out = sum(p for p, _ in reqs), sum(o for _, o in reqs)
+    stats = engine.cache_stats()
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": f"generated tok/s, continuous batching of {args.serve} requests ({shape_name} shape, {dkey})",
+        "value": round(t_out / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(dt * 1e3 / steps, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dkey, "data": "synthetic (uniform-random token ids and lengths, random weights N(0, 0.02))",
+        "config": {"model": f"{shape_name} shape", "layers": raw["num_hidden_layers"], "requests": args.serve,
+                   "prompt_tokens": t_in, "generated_tokens": t_out, "step_budget": 2048, "max_num_seqs": max_seqs,
+                   "cache_blocks": num_blocks, "block_size": block, "parallelism": "single GPU"},
+        "total_tok_s": round((t_in + t_out) / dt, 1), "seconds": round(dt, 3),
+        "preemptions": stats["preemptions"], "held_back": stats["held_back"], "tokens_computed": stats["tokens"],
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,6 +180,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--serve", type=int, default=0, metavar="REQUESTS",
+                    help="instead of the decode measurement: continuous batching of this many requests")
+    ap.add_argument("--num-blocks", type=int, default=None, help="with --serve: cache blocks (default: room for all)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -148,6 +203,8 @@ def main() -> int:
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
+    if args.serve:
+        return serve_run(args, raw, shape_name)
     cfg = config_from_dict(raw)
     ctx_len = raw["max_position_embeddings"]
     max_batch = max(args.batch, 1 if args.no_points else 64)

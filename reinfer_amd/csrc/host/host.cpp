@@ -26,12 +26,14 @@
 #include <pybind11/stl.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstring>
 #include <deque>
 #include <memory>
 #include <string>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 namespace py = pybind11;
@@ -611,13 +613,23 @@ struct Scheduler {
   std::vector<RequestP> running;
   std::unordered_map<py::object, RequestP, KeyHash, KeyEq> requests;
   long arrivals = 0;
-  long c_steps = 0, c_preemptions = 0, c_finished = 0, c_refused = 0, c_tokens = 0;
+  long c_steps = 0, c_preemptions = 0, c_finished = 0, c_refused = 0, c_tokens = 0, c_held_back = 0;
+  // Admission by estimate (crates/scheduler/src/admission.rs:1-27): a request is let in only while the
+  // peak of what the running set is expected to hold fits the pool. Without it ("blocks") a request is
+  // let in as soon as its first portion's blocks are free, and a full pool preempts its way out.
+  bool peak_admission = true;
+  double ema_out = 2048.0;                  // output length of finished requests (admission.rs:34-37)
+  static constexpr double EMA_FLOOR = 64.0, BUSY_RATIO = 0.8;     // sched_loop.rs:749
+  static constexpr int ADDED_OUTPUT_LEN = 16;                     // admission.rs:31
 
   Scheduler(std::shared_ptr<CacheManager> m, int max_num_seqs_, int max_num_batched_tokens, int max_model_len_,
-            py::object max_chunk_, std::vector<int> eos_ids)
+            py::object max_chunk_, std::vector<int> eos_ids, const std::string& admission)
       : manager(std::move(m)), budget(max_num_batched_tokens), max_model_len(max_model_len_), eos(std::move(eos_ids)) {
     if (max_num_seqs_ < 1 || max_num_batched_tokens < 1)
       throw py::value_error("max_num_seqs and max_num_batched_tokens must be positive");
+    if (admission != "peak" && admission != "blocks")
+      throw py::value_error("admission is \"peak\" (by the estimated peak of the running set) or \"blocks\" (by free blocks alone)");
+    peak_admission = admission == "peak";
     max_num_seqs = std::min(max_num_seqs_, manager->slots.num_slots);
     max_chunk = (max_chunk_.is_none() || max_chunk_.cast<int>() <= 0) ? max_num_batched_tokens : max_chunk_.cast<int>();
   }
@@ -682,6 +694,56 @@ struct Scheduler {
     return true;
   }
   bool has_work() const { return !waiting.empty() || !running.empty(); }
+
+  // (a, b) of a request: a = tokens it holds once its current tokens are in the cache, plus one;
+  // b = new tokens it is expected to add yet: all it may when the pool is busy, else up to the
+  // larger of 1.1 x what it has generated and the running mean of finished requests' lengths, plus a
+  // slack of 16 (admission.rs:72-86; the reference counts the generated tokens in a and again in b,
+  // here b is what is still to come; its term for steps that a portioned prompt waits between
+  // portions is left out: no step here runs without the waiting portions).
+  std::pair<long, long> estimate(const Request& r, bool busy) const {
+    const long gen = (long)r.output.size();
+    const long a = (long)r.num_tokens() + 1;
+    long total = r.max_tokens;
+    if (!busy) total = std::min<long>(total, std::max<long>((long)std::ceil(1.1 * gen), (long)ema_out));
+    total = std::min<long>(total, std::max(0, max_model_len - (int)r.prompt.size()));
+    return {a, std::max<long>(0, total - gen) + ADDED_OUTPUT_LEN};
+  }
+  // The most tokens the set will hold at one time if every request adds its b and then leaves: sorted
+  // by b descending, max over k of b[k] * (k + 1) + a[0] + ... + a[k] (admission.rs:138-148).
+  static long peak_tokens(std::vector<std::pair<long, long>> set) {
+    std::stable_sort(set.begin(), set.end(), [](const std::pair<long, long>& x, const std::pair<long, long>& y) { return x.second > y.second; });
+    long peak = 0, cur = 0;
+    for (size_t k = 0; k < set.size(); ++k) {
+      cur += set[k].first;
+      peak = std::max(peak, set[k].second * (long)(k + 1) + cur);
+    }
+    return peak;
+  }
+  bool busy() const {
+    double worst = 0.0;
+    for (auto& p : manager->pools)
+      worst = std::max(worst, 1.0 - (double)p.num_free() / std::max(1, p.num_blocks));
+    return worst >= BUSY_RATIO;
+  }
+  // May `cand` join `set` (estimates of the running requests)? Busy: everything at once must fit;
+  // otherwise the peak must (admission.rs:211-240). A request's last block may be partly empty.
+  bool estimate_admits(const std::vector<std::pair<long, long>>& set, const std::pair<long, long>& cand, bool is_busy) const {
+    std::vector<std::pair<long, long>> all(set);
+    all.push_back(cand);
+    const long pool = (long)pool_tokens() - (long)all.size() * (manager->block_size - 1);
+    if (is_busy) {
+      long sum = 0;
+      for (auto& e : all) sum += e.first + e.second;
+      if (sum > pool) return false;
+    }
+    return peak_tokens(std::move(all)) <= pool;
+  }
+  void observe_output(long n) {
+    // running mean of output lengths: slow to fall, quicker to rise, never below 64 (admission.rs:113-126)
+    const double alpha = (double)n > ema_out ? 0.9 : 0.6;
+    ema_out = std::max(EMA_FLOOR, alpha * ema_out + (1.0 - alpha) * (double)n);
+  }
 
   void preempt(const RequestP& req, StepPlan& plan) {
     running.erase(std::find(running.begin(), running.end(), req));
@@ -779,10 +841,24 @@ struct Scheduler {
     }
 
     // 3. admissions: resumed first (they sit at the head), then arrival order
+    std::vector<std::pair<long, long>> working;
+    const bool is_busy = peak_admission && busy();
+    if (peak_admission && !waiting.empty())
+      for (auto& r : running) working.push_back(estimate(*r, is_busy));
     while (!waiting.empty() && left > 0 && (int)running.size() < max_num_seqs) {
       auto r = waiting.front();
       if (std::find(plan.preempted.begin(), plan.preempted.end(), r) != plan.preempted.end())
         break;                      // preempted in this very step: not before the next
+      if (peak_admission && !running.empty()) {      // a lone request always runs: add() saw that it can fit
+        const auto e = estimate(*r, is_busy);
+        if (!estimate_admits(working, e, is_busy)) {
+          ++c_held_back;
+          break;
+        }
+        working.push_back(e);
+      } else if (peak_admission) {
+        working.push_back(estimate(*r, is_busy));
+      }
       // a block of headroom for every running request, so that an admission does not force a
       // preemption at the very next step
       const int n = fit(r, 0, std::min({r->remaining(), max_chunk, left}), false, (int)running.size());
@@ -850,6 +926,7 @@ struct Scheduler {
         running.erase(std::find(running.begin(), running.end(), r));
         manager->free(r->rid);
         ++c_finished;
+        observe_output((long)r->output.size());
         done.push_back(r);
       }
     }
@@ -896,6 +973,7 @@ struct Scheduler {
     d["finished"] = c_finished;
     d["refused"] = c_refused;
     d["tokens"] = c_tokens;
+    d["held_back"] = c_held_back;
     return d;
   }
 };
@@ -1022,9 +1100,15 @@ PYBIND11_MODULE(_host, m) {
       .def_property_readonly("num_tokens", &StepPlan::num_tokens);
 
   py::class_<Scheduler>(m, "Scheduler")
-      .def(py::init<std::shared_ptr<CacheManager>, int, int, int, py::object, std::vector<int>>(), py::arg("manager"),
-           py::kw_only(), py::arg("max_num_seqs"), py::arg("max_num_batched_tokens"), py::arg("max_model_len"),
-           py::arg("max_chunk") = py::none(), py::arg("eos_token_ids") = std::vector<int>())
+      .def(py::init<std::shared_ptr<CacheManager>, int, int, int, py::object, std::vector<int>, const std::string&>(),
+           py::arg("manager"), py::kw_only(), py::arg("max_num_seqs"), py::arg("max_num_batched_tokens"),
+           py::arg("max_model_len"), py::arg("max_chunk") = py::none(), py::arg("eos_token_ids") = std::vector<int>(),
+           py::arg("admission") = "peak")
+      .def_readonly("peak_admission", &Scheduler::peak_admission)
+      .def_readonly("ema_out", &Scheduler::ema_out)
+      .def("estimate", [](const Scheduler& s, const RequestP& r, bool busy) { return s.estimate(*r, busy); }, py::arg("request"), py::arg("busy") = false)
+      .def_static("peak_tokens", &Scheduler::peak_tokens, py::arg("estimates"))
+      .def("observe_output", &Scheduler::observe_output, py::arg("length"))
       .def_readonly("manager", &Scheduler::manager)
       .def_readonly("max_num_seqs", &Scheduler::max_num_seqs)
       .def_readonly("budget", &Scheduler::budget)

@@ -42,7 +42,7 @@ class LLMEngine:
                  max_model_len: Optional[int] = None, block_size: int = 16,
                  num_blocks: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, max_chunk: Optional[int] = None,
-                 memory_fraction: float = 0.9):
+                 memory_fraction: float = 0.9, admission: str = "peak"):
         limits = dict(block_size=block_size, num_blocks=num_blocks, max_seqs=max_num_seqs,
                       max_model_len=max_model_len, memory_fraction=memory_fraction)
         if model is not None:
@@ -59,7 +59,7 @@ class LLMEngine:
         self.scheduler = Scheduler(self.runner.manager, max_num_seqs=max_num_seqs,
                                    max_num_batched_tokens=max_num_batched_tokens,
                                    max_model_len=self.runner.max_model_len, max_chunk=max_chunk,
-                                   eos_token_ids=self.runner.spec.eos_token_ids)
+                                   eos_token_ids=self.runner.spec.eos_token_ids, admission=admission)
         self.sampler = Sampler(self.device)
         self._auto_id = 0
         self.timings: Dict[str, float] = {}

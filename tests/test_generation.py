@@ -31,11 +31,16 @@ def check_greedy(folder, device):
     assert [o.token_ids for o in outs] == want
     assert all(o.finish_reason == "length" for o in outs)
     # so few blocks that requests are preempted and recomputed: the same tokens
-    small = engine_for(folder, device, num_blocks=6, max_num_batched_tokens=24)
+    small = engine_for(folder, device, num_blocks=6, max_num_batched_tokens=24, admission="blocks")
     outs2 = small.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16))
     assert [o.token_ids for o in outs2] == want
     assert small.cache_stats()["preemptions"] > 0
     assert small.cache_stats()["blocks_free"] == small.cache_stats()["blocks_total"]
+    # the same pool with admission by the estimated peak: requests wait instead, nothing is recomputed
+    held = engine_for(folder, device, num_blocks=6, max_num_batched_tokens=24)
+    outs3 = held.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16))
+    assert [o.token_ids for o in outs3] == want
+    assert held.cache_stats()["preemptions"] == 0 and held.cache_stats()["held_back"] > 0
     return eng
 
 

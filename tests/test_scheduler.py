@@ -9,11 +9,12 @@ from reinfer_amd.engine.scheduler import FINISHED, RUNNING, WAITING, RequestRefu
 from reinfer_amd.sampling import SamplingParams
 
 
-def make(num_blocks=64, bs=4, max_seqs=8, budget=32, max_model_len=512, max_chunk=None, eos=(), windows=(0,)):
+def make(num_blocks=64, bs=4, max_seqs=8, budget=32, max_model_len=512, max_chunk=None, eos=(), windows=(0,),
+         admission="blocks"):
     groups = [CacheGroupSpec(window=w, entries=(i,)) for i, w in enumerate(windows)]
     m = CacheManager(groups, bs, [num_blocks] * len(groups), max_seqs)
     s = Scheduler(m, max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_model_len,
-                  max_chunk=max_chunk, eos_token_ids=eos)
+                  max_chunk=max_chunk, eos_token_ids=eos, admission=admission)
     return m, s
 
 
@@ -246,3 +247,90 @@ def test_stop_sequences_fire_on_the_generated_suffix():
     assert run([6, 4, 2], ((), (4,))) == ([6], "stop")
     # the prompt's tokens do not count: 3 1 in the prompt, 4 generated first
     assert run([4, 3, 1, 4, 0], ((3, 1, 4),), prompt=(3, 1)) == ([4, 3, 1], "stop")
+
+
+# ---------------------------------------------------------------- admission by the estimated peak
+def test_peak_formula_and_estimates():
+    """max over k of b[k] (k + 1) + a[0..k], sorted by b descending (crates/scheduler/src/admission.rs:138-148):
+    the cases are worked by hand."""
+    assert Scheduler.peak_tokens([]) == 0
+    assert Scheduler.peak_tokens([(10, 5)]) == 15
+    # b descending: (10, 30), (100, 20), (50, 1): 30 + 10 = 40; 20 * 2 + 110 = 150; 1 * 3 + 160 = 163
+    assert Scheduler.peak_tokens([(100, 20), (50, 1), (10, 30)]) == 163
+    # one long request beside short ones: the peak is while all are there, not the sum of all ends
+    assert Scheduler.peak_tokens([(10, 100), (10, 2), (10, 2)]) == max(100 + 10, 2 * 2 + 20, 2 * 3 + 30)
+    m, s = make(num_blocks=1024, bs=4, max_model_len=4096, admission="peak")
+    r = s.add("a", [1] * 20, SamplingParams(max_tokens=300), seed=0)
+    assert s.ema_out == 2048.0
+    assert s.estimate(r) == (21, 300 + 16)                 # not busy: min(cap, max(1.1 * 0, mean)) + 16
+    s.observe_output(100)                                   # falls with weight 0.4 on what was seen
+    assert abs(s.ema_out - (0.6 * 2048 + 0.4 * 100)) < 1e-9
+    for _ in range(40):
+        s.observe_output(10)
+    assert s.ema_out == 64.0                                # never below 64
+    assert s.estimate(r) == (21, 64 + 16)
+    assert s.estimate(r, busy=True) == (21, 300 + 16)       # busy: all it may
+    while len(r.output) < 100:
+        run_step(m, s)
+    import math
+    assert s.estimate(r) == (121, math.ceil(1.1 * 100) - 100 + 16)      # 1.1 x what it has generated, less what it has
+    s.observe_output(1000)                                  # rises with weight 0.1
+    assert abs(s.ema_out - (0.9 * 64 + 0.1 * 1000)) < 1e-9
+
+
+def test_peak_admission_holds_back_instead_of_preempting():
+    """64 tokens of cache for three requests of about 39: admitted by blocks they preempt each
+    other; admitted by the estimate they run one after the other, nothing is recomputed, and the
+    outputs are the same. Arrival order is kept: nobody overtakes the request that is held back."""
+    def run(admission):
+        m, s = make(num_blocks=16, bs=4, budget=64, max_seqs=4, admission=admission)
+        for i, n in enumerate([9, 7, 8]):
+            s.add(f"r{i}", list(range(1, n + 1)), SamplingParams(max_tokens=30), seed=i)
+        log = []
+        outs = drive(m, s, log)
+        assert all(p.num_free == p.num_blocks for p in m.pools)
+        return outs, log, s
+    by_blocks, _, s_blocks = run("blocks")
+    by_peak, log, s_peak = run("peak")
+    assert by_peak == by_blocks
+    assert s_blocks.counters["preemptions"] > 0
+    assert s_peak.counters["preemptions"] == 0 and s_peak.counters["held_back"] > 0
+    assert s_peak.counters["tokens"] == sum(n + 29 for n in (9, 7, 8)), "every token computed once"
+    first_seen = []
+    for portions, _ in log:
+        for rid, _, _ in portions:
+            if rid not in first_seen:
+                first_seen.append(rid)
+    assert first_seen == ["r0", "r1", "r2"]
+
+
+def test_peak_admission_lets_in_what_fits_and_a_lone_request_always():
+    m, s = make(num_blocks=64, bs=4, budget=256, max_seqs=8, admission="peak")      # 256 tokens
+    for _ in range(8):
+        s.observe_output(8)                                 # the mean of finished outputs comes down to its floor of 64
+    for i in range(4):
+        s.add(f"r{i}", [1] * 20, SamplingParams(max_tokens=40), seed=i)
+    plan, _ = run_step(m, s)
+    # (a, b) = (21, 56) each; the pool less a partly empty block a request: k requests need 56 k + 21 k + 3 k <= 256
+    assert [p.request.rid for p in plan.portions] == ["r0", "r1", "r2"]
+    assert s.counters["held_back"] == 1
+    # a request larger than the estimate allows still runs when it is alone
+    m2, s2 = make(num_blocks=16, bs=4, budget=64, admission="peak")
+    s2.add("big", [1] * 30, SamplingParams(max_tokens=500), seed=0)
+    plan, _ = run_step(m2, s2)
+    assert [(p.request.rid, p.length) for p in plan.portions] == [("big", 30)]
+
+
+def test_peak_admission_is_deterministic_and_complete():
+    import random
+    def run():
+        rng = random.Random(5)
+        m, s = make(num_blocks=40, bs=4, budget=48, max_seqs=6, admission="peak")
+        for i in range(30):
+            s.add(f"r{i}", [1 + i] * rng.randint(1, 60), SamplingParams(max_tokens=rng.randint(1, 40)), seed=i)
+        log = []
+        outs = drive(m, s, log)
+        return outs, log, dict(s.counters)
+    a, b = run(), run()
+    assert a == b
+    assert len(a[0]) == 30 and all(reason == "length" for _, reason in a[0].values())
