@@ -18,6 +18,7 @@ The reference launches every kernel of every step from the host
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -128,8 +129,19 @@ class _CapturedStep:
         cur.wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, pool=pool), torch.no_grad():
-            self._body()
+        # No garbage collection inside the capture: a dead cycle that holds device memory or a graph
+        # of its own (an earlier runner with its captured steps) would be destroyed in the middle of
+        # it, and releasing device memory while a stream captures is an error that ends the process.
+        # Such cycles are collected here, before the capture begins.
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph, pool=pool), torch.no_grad():
+                self._body()
+        finally:
+            if was_enabled:
+                gc.enable()
 
     def fill(self, entries: List[StepEntry], sampling) -> None:
         self.rows.fill(entries, self.h, sampling)

@@ -192,3 +192,30 @@ def test_decode_graphs_replay_like_eager_steps(folders, which, n_req):
     assert len(keys) >= 2
     if which == "B":                                      # 70 and 68 requests pad to 80 rows; 512 is the second context bucket
         assert {(80, 256), (80, 512)} <= keys
+
+
+def test_no_garbage_collection_inside_a_capture(folders):
+    """A runner that is dropped is a dead cycle holding captured graphs and their memory. Were it
+    collected while the next runner captures a step, its memory would be released in the middle of
+    the capture, which ends the process. The capture collects such cycles first and keeps the
+    collector off until it is over: here the collector is set to run at every allocation."""
+    import gc
+    dtype, which = "bfloat16", "A"
+    V = vocab(which)
+    toks = random_tokens(40, V, 77)
+    old = gc.get_threshold()
+
+    def decode_some():
+        runner = runner_for(folders, which, dtype, max_tokens=256)
+        got = run_plan(runner, {"r": toks}, [[("r", 30)]] + [[("r", 1)]] * 10)["r"]
+        assert runner.graphs is not None and runner.graphs.replays >= 10
+        return got
+
+    first = decode_some()                       # its runner is garbage from here on (a cycle: not freed by counting)
+    gc.set_threshold(1, 1, 1)
+    try:
+        second = decode_some()
+        assert gc.isenabled()
+    finally:
+        gc.set_threshold(*old)
+    assert torch.equal(first, second)

@@ -639,6 +639,22 @@ def test_linear_dispatch_refuses_nothing_silently():
                             torch.empty(65, 8, device=DEV, dtype=torch.bfloat16))
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 1003, 200), (130, 333, 72), (300, 5001, 264)])
+def test_linear_float_result_from_bfloat16_above_64_rows(M, N, K):
+    """The head's logits for more than 64 wanted rows: float out of bfloat16 operands, summed in
+    float (a rounded bfloat16 result would be off by 2^-9 of the value), 64 rows at a time
+    through the weight-streaming kernel; a row stride it does not take goes to the plain kernel."""
+    g = torch.Generator(device="cpu").manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(DEV).to(torch.bfloat16)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops().linear(x, w, out)
+    close(out, x.double() @ w.double().T, 2e-5)
+    odd = torch.randn(M, K + 1, generator=g).to(DEV).to(torch.bfloat16)[:, :K]      # row stride K + 1
+    ops().linear(odd, w, out)
+    close(out, odd.double() @ w.double().T, 2e-5)
+
+
 DEC_SHAPES = [(4, 2, 16), (14, 2, 64), (12, 2, 48), (5, 5, 32), (8, 1, 128), (32, 8, 128), (2, 1, 256), (6, 3, 80)]
 DEC_BATCHES = [
     ([1], [0]), ([1], [15]), ([1], [16]), ([1, 1, 1], [31, 32, 700]), ([1] * 5, [63, 64, 65, 1000, 2]),
