@@ -198,24 +198,35 @@ def test_no_garbage_collection_inside_a_capture(folders):
     """A runner that is dropped is a dead cycle holding captured graphs and their memory. Were it
     collected while the next runner captures a step, its memory would be released in the middle of
     the capture, which ends the process. The capture collects such cycles first and keeps the
-    collector off until it is over: here the collector is set to run at every allocation."""
+    collector off until it is over: here the collector is set to run at every allocation, and the
+    forward pass notes whether it is on whenever the stream is capturing."""
     import gc
     dtype, which = "bfloat16", "A"
     V = vocab(which)
     toks = random_tokens(40, V, 77)
     old = gc.get_threshold()
+    seen = []
 
-    def decode_some():
+    def decode_some(watch):
         runner = runner_for(folders, which, dtype, max_tokens=256)
+        if watch:
+            forward = runner.model.forward
+
+            def noting(*a, **k):
+                if torch.cuda.is_current_stream_capturing():
+                    seen.append(gc.isenabled())
+                return forward(*a, **k)
+            runner.model.forward = noting
         got = run_plan(runner, {"r": toks}, [[("r", 30)]] + [[("r", 1)]] * 10)["r"]
         assert runner.graphs is not None and runner.graphs.replays >= 10
         return got
 
-    first = decode_some()                       # its runner is garbage from here on (a cycle: not freed by counting)
+    first = decode_some(False)                  # its runner is garbage from here on (a cycle: not freed by counting)
     gc.set_threshold(1, 1, 1)
     try:
-        second = decode_some()
+        second = decode_some(True)
         assert gc.isenabled()
     finally:
         gc.set_threshold(*old)
+    assert seen and not any(seen), "the collector must be off while a step is captured"
     assert torch.equal(first, second)
