@@ -67,13 +67,13 @@ def kv_bytes_per_token(raw: dict, elem: int) -> int:
     return 2 * raw["num_hidden_layers"] * raw["num_key_value_heads"] * raw["head_dim"] * elem
 
 
-def decode_run(engine, raw, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
+def decode_run(engine, raw, batch: int, prompt_len: int, steps: int, warmup: int, seed: int, max_tokens: int):
     """Prefill ``batch`` prompts, then time ``steps`` decode steps. -> (ms a step, mean context)."""
     import torch
     from reinfer_amd.sampling import SamplingParams
     g = torch.Generator().manual_seed(seed)
-    params = SamplingParams(temperature=0.0, max_tokens=raw["max_position_embeddings"] - prompt_len - 1,
-                            ignore_eos=True)
+    # the cap on new tokens is what the run needs: the scheduler admits by what requests may come to hold
+    params = SamplingParams(temperature=0.0, max_tokens=max_tokens, ignore_eos=True)
     rids = []
     for _ in range(batch):
         ids = torch.randint(0, raw["vocab_size"], (prompt_len,), generator=g).tolist()
@@ -183,6 +183,8 @@ def main() -> int:
     ap.add_argument("--serve", type=int, default=0, metavar="REQUESTS",
                     help="instead of the decode measurement: continuous batching of this many requests")
     ap.add_argument("--num-blocks", type=int, default=None, help="with --serve: cache blocks (default: room for all)")
+    ap.add_argument("--max-model-len", type=int, default=None, metavar="N",
+                    help="context length (default: the shape's: 4096 at 8b, 8192 at 4b, 16384 at 32b)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the Qwen3-8B shape)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -203,19 +205,28 @@ def main() -> int:
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
+    if args.max_model_len:
+        raw["max_position_embeddings"] = args.max_model_len
     if args.serve:
         return serve_run(args, raw, shape_name)
     cfg = config_from_dict(raw)
     ctx_len = raw["max_position_embeddings"]
     max_batch = max(args.batch, 1 if args.no_points else 64)
     block = 16
-    # a request decodes while later prompts are still being prefilled: one step a prompt
-    blocks_per_req = -(-(args.prompt_len + max_batch + args.warmup + args.steps + 16) // block)
+    # a request decodes while later prompts are still being prefilled: one step a portion of a prompt
+    budget = max(2048, args.prefill_tokens)
+    prompt_steps = max_batch * -(-args.prompt_len // budget)
+    if args.prompt_len + prompt_steps + args.warmup + args.steps + 16 > ctx_len:
+        print(f"bench.py: {max_batch} prompts of {args.prompt_len} tokens and {args.warmup + args.steps} decode steps "
+              f"do not fit a context of {ctx_len}", file=sys.stderr)
+        return 2
+    max_new = prompt_steps + args.warmup + args.steps + 16
+    blocks_per_req = -(-(args.prompt_len + max_new + 32) // block) + 1
     num_blocks = max_batch * blocks_per_req + 8
     log(f"building {raw['num_hidden_layers']} layers of the {shape_name} shape in {args.dtype}, random weights ...")
     t0 = time.perf_counter()
     engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=block, num_blocks=num_blocks,
-                       max_num_seqs=max_batch, max_num_batched_tokens=max(2048, args.prefill_tokens),
+                       max_num_seqs=max_batch, max_num_batched_tokens=budget,
                        max_model_len=ctx_len)
     torch.cuda.synchronize()
     log(f"model ready in {time.perf_counter() - t0:.1f} s; {num_blocks} cache blocks of {block}")
@@ -236,7 +247,7 @@ def main() -> int:
                "frac": round(pf_flops / (pf_ms * 1e-3) / MFMA_PEAK[dkey], 4)}
     log(f"prefill {T} tokens: {pf_ms:.2f} ms, {prefill['value']:.0f} tok/s, {prefill['frac']:.3f} of the MFMA peak")
 
-    ms, ctx = decode_run(engine, raw, args.batch, args.prompt_len, args.steps, args.warmup, args.seed + 2)
+    ms, ctx = decode_run(engine, raw, args.batch, args.prompt_len, args.steps, args.warmup, args.seed + 2, max_new)
     value = args.batch / (ms * 1e-3)
     step_bytes = n_lin * elem + args.batch * ctx * kv_tok
     achieved = step_bytes / (ms * 1e-3)
@@ -246,7 +257,7 @@ def main() -> int:
     if not args.no_points:
         for b in (1, 64):
             steps_b = args.steps if b == 1 else max(16, args.steps // 2)
-            pms, _ = decode_run(engine, raw, b, args.prompt_len, steps_b, min(args.warmup, 16), args.seed + 3 + b)
+            pms, _ = decode_run(engine, raw, b, args.prompt_len, steps_b, min(args.warmup, 16), args.seed + 3 + b, max_new)
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
             log(f"decode batch {b}: {pms:.3f} ms a step, {points[f'decode_b{b}']:.0f} tok/s")
 
