@@ -53,3 +53,41 @@ def test_trace_run_mixed_steps(tmp_path, dtype):
             continue
         got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(len(want_rows), V))
         assert rel_err(got, torch.stack(want_rows)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("which,dtype", [("C", "float32"), ("B", "bfloat16")])
+def test_trace_run_orders_ids_and_idle_requests(tmp_path, which, dtype):
+    """What a trace may do beside the plain cases: ``want`` in any order and with a place twice, an
+    entry of a decode step that wants nothing, a step in which nothing is wanted at all (no file), a
+    request left out of steps and going on later, a request that ends while idle, an id that is a
+    number, and an id used again after its end (a fresh request on used blocks)."""
+    folder = make_folder(tmp_path, which, dtype)
+    raw, weights = read_folder(folder)
+    V = raw["vocab_size"]
+    a, b, c, a2 = (random_tokens(n, V, s) for n, s in ((40, 1), (30, 2), (20, 3), (25, 4)))
+    ra, rb, ra2 = (plain.forward(raw, weights, t).float() for t in (a, b, a2))
+    steps = [
+        ({"step": 0, "entries": [{"id": "a", "tokens": a[:10], "want": [9, 0, 3]},
+                                 {"id": 7, "tokens": b[:2], "want": []}], "end": []}, ra[[9, 0, 3]]),
+        ({"step": 1, "entries": [{"id": "a", "tokens": a[10:11], "want": []},
+                                 {"id": 7, "tokens": b[2:3], "want": [0]}], "end": []}, rb[[2]]),
+        ({"step": 2, "entries": [{"id": 7, "tokens": b[3:30], "want": [26, 26, 0]}], "end": []}, rb[[29, 29, 3]]),
+        ({"step": 3, "entries": [{"id": "c", "tokens": c, "want": []}], "end": [7]}, None),
+        ({"step": 4, "entries": [{"id": "a", "tokens": a[11:40], "want": [28]}], "end": ["a", "c"]}, ra[[39]]),
+        ({"step": 5, "entries": [{"id": "a", "tokens": a2[:24], "want": [23]}], "end": []}, ra2[[23]]),
+        ({"step": 6, "entries": [{"id": "a", "tokens": a2[24:25], "want": [0]}], "end": ["a"]}, ra2[[24]]),
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "192"],
+        input="".join(json.dumps(s) + "\n" for s, _ in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(7)]
+    for s, ref in steps:
+        path = out / f"{s['step']}.f32"
+        if ref is None:
+            assert not path.exists()
+            continue
+        got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(ref.shape[0], V))
+        assert rel_err(got, ref) < TOL[dtype], s["step"]
