@@ -248,11 +248,14 @@ class HipKernels:
 
     def _attention_plan(self, batch, device, tile: int, room: int = 0):
         """Which tokens go to which kernel; made once per step and query-tile size,
-        shared by the layers. With fewer than ``room`` query tiles (workgroups for less than
-        the whole chip), the tiles with the most keys are listed twice, each time with half of
-        the heads, as many as there is room for: the prompt kernel lasts as long as its heaviest
-        tile (measured at 1024 tokens, 32 heads of 128: 45 -> 37 us; with more tiles than CUs the
-        second workgroups would only queue behind the first: 85 -> 113 us at 2048 tokens)."""
+        shared by the layers. ``room`` is the number of query tiles whose workgroups fill the
+        chip once. With up to 5/4 of that, the tiles with the most keys are listed twice, each
+        time with half of the heads: the prompt kernel lasts as long as its heaviest tile, and a
+        half tile that queues behind a light one still ends before a whole heavy one would. Below
+        ``room`` tiles as many as there is room for, and at least a quarter of ``room``; from
+        ``room`` to 5/4 of it 3/16 of ``room`` (measured with 32 heads of 128 over 8 groups, room
+        32: 1024 tokens 45 -> 37 us, 1792: 65 -> 61, 2048: 84 -> 71, 2304: 94 -> 83, 2560: 104 -> 96;
+        at 3072 tokens, 48 tiles, any second listing is slower)."""
         plan = batch.extra.get("attention_plan")
         if plan is not None and plan.get("tile", tile) == tile:
             return plan
@@ -277,9 +280,14 @@ class HipKernels:
             # the longest of every request start first, whatever the order of the requests
             quads = sorted((tuple(tiles[4 * k:4 * k + 4]) for k in range(n_tiles)), key=lambda t: t[3] + t[2])
             tiles = [v for t in quads for v in t]
-        if 0 < n_tiles < room:
+        n_twice = 0
+        if 0 < n_tiles <= room:
+            n_twice = min(n_tiles, max(room - n_tiles, room // 4))
+        elif room < n_tiles <= room + room // 4:
+            n_twice = (3 * room) // 16
+        if n_twice:
             by_keys = sorted(range(n_tiles), key=lambda k: -(tiles[4 * k + 3] + tiles[4 * k + 2]))
-            twice = set(by_keys[:room - n_tiles])
+            twice = set(by_keys[:n_twice])
             cut = []
             for k in range(n_tiles):
                 i, row, n, pos = tiles[4 * k:4 * k + 4]
