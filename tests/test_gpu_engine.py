@@ -230,3 +230,28 @@ def test_no_garbage_collection_inside_a_capture(folders):
         gc.set_threshold(*old)
     assert seen and not any(seen), "the collector must be off while a step is captured"
     assert torch.equal(first, second)
+
+
+@pytest.mark.parametrize("which,dtype", [("B", "bfloat16"), ("C", "bfloat16"), ("A", "float32")])
+def test_many_decoding_requests_beside_prompt_portions(folders, plain_cache, which, dtype):
+    """Ten requests decode while two more are prefilled in portions: in bfloat16 such a step runs the
+    decode attention on a second stream beside the prompt attention; both write rows of one output."""
+    V = vocab(which)
+    seqs = {f"d{i}": random_tokens(30 + 3 * i, V, 500 + i) for i in range(10)}
+    seqs["p"] = random_tokens(120, V, 600)
+    seqs["q"] = random_tokens(75, V, 601)
+    runner = runner_for(folders, which, dtype, max_tokens=64 * 16)
+    dec = [r for r in seqs if r.startswith("d")]
+    plan = [[(r, len(seqs[r]) - 12) for r in dec]]                          # the decoders' prompts, less 12 tokens
+    cuts_p, cuts_q = [40, 33, 5, 30, 12], [20, 2, 41, 12]
+    for step in range(12):
+        items = [(r, 1) for r in dec]
+        if step < len(cuts_p):
+            items.append(("p", cuts_p[step]))
+        if 2 <= step < 2 + len(cuts_q):
+            items.insert(3, ("q", cuts_q[step - 2]))
+        plan.append(items)
+    assert sum(cuts_p) == 120 and sum(cuts_q) == 75
+    got = run_plan(runner, seqs, plan)
+    for r, toks in seqs.items():
+        assert rel_err(got[r], reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype], r
