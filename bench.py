@@ -261,6 +261,10 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
             log(f"decode batch {b}: {pms:.3f} ms a step, {points[f'decode_b{b}']:.0f} tok/s")
 
+    peaks = kernels.current().measure_peaks(engine.device)
+    log(f"measured on this GPU: a plain read {peaks['hbm_read_GBps']:.0f} GB/s, bfloat16 matrix cores "
+        f"{peaks['mfma_bf16_32x32x16_TFLOPs']:.0f} TFLOP/s with 32x32x16 products, {peaks['mfma_bf16_16x16x32_TFLOPs']:.0f} with "
+        f"16x16x32 (nominal: {HBM_PEAK / 1e9:.0f} GB/s, {MFMA_PEAK['bf16'] / 1e12:.0f} TFLOP/s)")
     out = {
         "metric": f"decode tok/s at batch {args.batch} ({shape_name} shape, {dkey}, {args.prompt_len}-token prompts)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -279,6 +283,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        # what this GPU gives at best, beside the published peaks that the fractions above use
+        "measured_peaks": {k: round(v, 1) for k, v in peaks.items()},
     }
     print(json.dumps(out), flush=True)
     return 0

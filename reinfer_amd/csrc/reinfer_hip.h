@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 13
+#define RA_ABI_VERSION 14
 
 #ifdef __cplusplus
 extern "C" {
@@ -126,6 +126,14 @@ int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const 
 // its logit bias as bias_len pairs (token id, float bits) from bias_off, each id once.
 int ra_filter_logits(float* logits, int n_rows, int vocab, int row_stride, const void* rows,
                      const int* window, hipStream_t stream);
+
+// What the machine gives at best (peaks.hip; for measurement, not on the product path): one read of
+// `bytes` of device memory, and `iters` iterations of bfloat16 matrix-core products on registers
+// (shape 16: eight 16x16x32 an iteration; shape 32: four 32x32x16) in `waves_per_cu` waves on every CU
+// (*flops: what all of them did). `sink` is 4 bytes of
+// device memory that is never written in practice.
+int ra_stream_read(const void* src, long bytes, void* sink, hipStream_t stream);
+int ra_mfma_loop(int shape, int iters, int waves_per_cu, void* sink, double* flops, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 
 class KernelLibraryError(RuntimeError):
@@ -45,6 +45,8 @@ _SIGNATURES = {
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
     "ra_filter_logits": [P, I, I, I, P, P, P],
+    "ra_stream_read": [P, c_long, P, P],
+    "ra_mfma_loop": [I, I, I, P, P, P],
 }
 
 

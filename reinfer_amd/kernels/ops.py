@@ -658,3 +658,36 @@ class HipKernels:
         win_t = torch.tensor(window or [0], dtype=torch.int32).to(logits.device)
         library.call("ra_filter_logits", logits.data_ptr(), n, V, logits.stride(0), rows_t.data_ptr(),
                      win_t.data_ptr(), _stream())
+
+    # ------------------------------------------------------------ measurement
+    def measure_peaks(self, device="cuda:0", read_bytes: int = 4 << 30) -> dict:
+        """What the machine gives at best: GB/s of a plain read of ``read_bytes`` of device memory
+        (more than the chip's caches hold) and TFLOP/s of bfloat16 matrix-core products on
+        registers, in both instruction shapes. For pricing measured kernels beside the published peaks; not on the product path."""
+        import ctypes
+        buf = torch.empty(read_bytes // 4, dtype=torch.int32, device=device).random_()
+        sink = torch.zeros(1, dtype=torch.int32, device=device)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+        def timed(fn, reps):
+            fn()
+            torch.cuda.synchronize(device)
+            best = float("inf")
+            for _ in range(reps):
+                e0.record()
+                fn()
+                e1.record()
+                torch.cuda.synchronize(device)
+                best = min(best, e0.elapsed_time(e1) * 1e-3)
+            return best
+
+        with torch.cuda.device(device):
+            t_read = timed(lambda: library.call("ra_stream_read", buf.data_ptr(), read_bytes, sink.data_ptr(), _stream()), 5)
+            out = {"hbm_read_GBps": read_bytes / t_read / 1e9}
+            for shape, name in ((32, "mfma_bf16_32x32x16_TFLOPs"), (16, "mfma_bf16_16x16x32_TFLOPs")):
+                flops = ctypes.c_double(0.0)
+                t = timed(lambda: library.call("ra_mfma_loop", shape, 10000, 16, sink.data_ptr(),
+                                               ctypes.byref(flops), _stream()), 3)
+                out[name] = flops.value / t / 1e12
+        del buf
+        return out
