@@ -255,3 +255,22 @@ def test_many_decoding_requests_beside_prompt_portions(folders, plain_cache, whi
     got = run_plan(runner, seqs, plan)
     for r, toks in seqs.items():
         assert rel_err(got[r], reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype], r
+
+
+@pytest.mark.parametrize("stored,run", [("float32", "bfloat16"), ("bfloat16", "float32"), ("float16", "bfloat16"),
+                                        ("float16", "float32")])
+def test_stored_dtype_differs_from_the_run_dtype(tmp_path, stored, run):
+    """A folder stored in one type and run in another: matrices are rounded to bfloat16 for the
+    bfloat16 run, widened for the 32-bit run (crates/cuda/src/engine.rs:6572-6598 converts every
+    stored type to its run type on the host). The plain implementation takes the stored values."""
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.weights import write_model_folder
+    raw, seed = TINY["B"]
+    folder = str(tmp_path / f"b_{stored}")
+    write_model_folder(config_from_dict(raw), seed, folder, dtype=stored)
+    rawr, weights = read_folder(folder)
+    toks = random_tokens(90, raw["vocab_size"], 55)
+    ref = plain.forward(rawr, weights, toks).float()
+    runner = ModelRunner.from_folder(folder, dtype=run, device="cuda:0", max_tokens=128)
+    got = run_plan(runner, {"r": toks}, [[("r", 70)], [("r", 2)]] + [[("r", 1)]] * 18)["r"]
+    assert rel_err(got, ref) < TOL[run]
