@@ -274,3 +274,23 @@ def test_stored_dtype_differs_from_the_run_dtype(tmp_path, stored, run):
     runner = ModelRunner.from_folder(folder, dtype=run, device="cuda:0", max_tokens=128)
     got = run_plan(runner, {"r": toks}, [[("r", 70)], [("r", 2)]] + [[("r", 1)]] * 18)["r"]
     assert rel_err(got, ref) < TOL[run]
+
+
+@pytest.mark.parametrize("which,dtype", [("B", "float32"), ("C", "bfloat16")])
+def test_thousands_of_tokens_of_context(tmp_path, which, dtype):
+    """4500 tokens: portions of 2048 with earlier context behind them, then single tokens over a
+    context that takes many chunks of the decode kernel and the 8192 bucket of the captured steps."""
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.weights import write_model_folder
+    raw = dict(TINY[which][0], max_position_embeddings=8192)
+    folder = str(tmp_path / "long")
+    write_model_folder(config_from_dict(raw), 3, folder, dtype=dtype)
+    rawr, weights = read_folder(folder)
+    n = 4500
+    toks = random_tokens(n, raw["vocab_size"], 9)
+    ref = plain.forward(rawr, weights, toks).float()
+    runner = ModelRunner.from_folder(folder, dtype=dtype, device="cuda:0", max_tokens=4544)
+    plan = [[("r", 2048)], [("r", 2048)], [("r", 340)]] + [[("r", 1)]] * 64
+    got = run_plan(runner, {"r": toks}, plan)["r"]
+    assert rel_err(got, ref) < TOL[dtype]
+    assert rel_err(got[-64:], ref[-64:]) < TOL[dtype]
