@@ -268,20 +268,35 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
   }
 }
 
-// How [M, N, K] is cut: waves a workgroup (8 or 6, 16 features each) and K ranges. With many features
+// How [M, N, K] is cut: waves a workgroup (5 to 8, 16 features each) and K ranges. With many features
 // one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
-// workgroups of 96). With few features 128 a workgroup and the smallest power of two up to 8 of K
+// workgroups of 96; 19456: 244 of 80; 51200: 458 of 112). With few features 128 a workgroup and the smallest power of two up to 8 of K
 // ranges that gives at least 192 workgroups, each range a multiple of the run and two runs or more.
-static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_split, bool* partial = nullptr,
+static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int* k_per_split, bool* partial = nullptr,
                      bool emits = false) {
   if (partial) *partial = emits;                       // the adding kernel writes what the next norm needs
-  const int cb8 = (N + 127) / 128, cb6 = (N + 95) / 96;
+  const int cb8 = (N + 127) / 128;
   *waves = 8;
   *S = 1;
   *k_per_split = (K + GW_KS - 1) / GW_KS * GW_KS;
   if ((cb8 >= 192 && !emits) || epilogue == WEPI_SILU_PAIRS) {
-    const double e8 = (double)cb8 / (((cb8 + 255) / 256) * 256), e6 = (double)cb6 / (((cb6 + 255) / 256) * 256);
-    if (e6 > e8) *waves = 6;
+    // The width whose workgroups fill whole rounds of the chip's 256 CUs best: 5 to 8 waves from 17 rows
+    // on, 6 or 8 below (there the odd widths were slower inside a decode step although faster alone, and
+    // a shape that neither 6 nor 8 fills well goes to gemm_skinny: ra_gemm_wide_preferred). A narrower
+    // workgroup stages the activations more often, so it must fill the rounds clearly better (with many
+    // rounds, as for a vocabulary, the widths differ little in that and the widest stays). Measured
+    // inside decode steps, against 6 or 8 waves at every row count: 51200 x 5120 gated, 64 layers: -4 % a step
+    // at 1 and 8 rows, -2 % at 64; 19456 x 2560, 36 layers: -1.7 % at 1 row, -1 % at 64.
+    double best = -1.0;
+    for (int wv = 8; wv >= 5; --wv) {
+      if (M <= 16 && (wv == 7 || wv == 5)) continue;
+      const int cb = (N + wv * 16 - 1) / (wv * 16);
+      const double e = (double)cb / (((cb + 255) / 256) * 256);
+      if (e > best * 1.03) {
+        best = e;
+        *waves = wv;
+      }
+    }
     return;
   }
   int s = 1;
@@ -299,10 +314,17 @@ static void gw_split(int epilogue, int N, int K, int* waves, int* S, int* k_per_
 extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
   if (M < 1 || M > 64) return 0;
   int waves, S, kps;
-  gw_split(epilogue, N, K, &waves, &S, &kps);
-  // below 17 rows only the gated product of a wide feed-forward: one K range, enough workgroups to fill
-  // the chip (measured at 4 to 16 rows, 24576 x 4096: 37 us against 39 to 42)
-  if (M < 17) return (epilogue == WEPI_SILU_PAIRS && S == 1 && (N + waves * 16 - 1) / (waves * 16) >= 192) ? 1 : 0;
+  gw_split(epilogue, M, N, K, &waves, &S, &kps);
+  // below 17 rows the gated product of a wide feed-forward: one K range, enough workgroups to fill the
+  // chip (measured at 4 to 16 rows, 24576 x 4096: 37 us against 39 to 42) and to fill whole rounds of it
+  // (400 workgroups would leave a third of the CUs with half the work: the other kernel's many small
+  // ones are then faster); and from 9 rows a plain product over a vocabulary (151936 features at 16 rows,
+  // K = 2560 / 4096 / 5120: 148 / 237 / 280 us against 170 / 239 / 327)
+  const int cb = (N + waves * 16 - 1) / (waves * 16);
+  if (M < 17) {
+    if (epilogue == WEPI_SILU_PAIRS) return (S == 1 && cb >= 192 && cb * 10 >= ((cb + 255) / 256) * 256 * 8) ? 1 : 0;
+    return (epilogue == WEPI_PLAIN && M > 8 && S == 1 && cb >= 768) ? 1 : 0;
+  }
   return (S == 1 || (long)N * K > 4096L * 4096L) ? 1 : 0;
 }
 
@@ -311,7 +333,7 @@ extern "C" long ra_gemm_wide_scratch(int epilogue, int M, int N, int K, int emit
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   int waves, S, kps;
   bool partial;
-  gw_split(epilogue, N, K, &waves, &S, &kps, &partial, emits != 0);
+  gw_split(epilogue, M, N, K, &waves, &S, &kps, &partial, emits != 0);
   return partial ? (long)S * M * N : 0;
 }
 
@@ -395,15 +417,15 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
            "gemm_wide: this product needs %ld floats of scratch, got %ld", need, scratch_floats);
   int waves, S, kps;
   bool partial;
-  gw_split(epilogue, N, K, &waves, &S, &kps, &partial, emits);
-#define RA_GWL(MT)                                                                                            \
-  return waves == 6 ? launch_wide<MT, 6>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream) \
-                    : launch_wide<MT, 8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream)
+  gw_split(epilogue, M, N, K, &waves, &S, &kps, &partial, emits);
+#define RA_GWW(MT, WV) launch_wide<MT, WV>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream)
+#define RA_GWL(MT) return waves == 5 ? RA_GWW(MT, 5) : waves == 6 ? RA_GWW(MT, 6) : waves == 7 ? RA_GWW(MT, 7) : RA_GWW(MT, 8)
   if (M <= 16) RA_GWL(1);
   if (M <= 32) RA_GWL(2);
   if (M <= 48) RA_GWL(3);
   RA_GWL(4);
 #undef RA_GWL
+#undef RA_GWW
 }
 
 // K ranges that ra_gemm_wide_partial cuts [M, N, K] into (its result has that many [M, N] float planes).
@@ -411,7 +433,7 @@ extern "C" int ra_gemm_wide_ranges(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   int waves, S, kps;
   bool partial;
-  gw_split(WEPI_PLAIN, N, K, &waves, &S, &kps, &partial, true);
+  gw_split(WEPI_PLAIN, M, N, K, &waves, &S, &kps, &partial, true);
   return S;
 }
 
@@ -426,18 +448,14 @@ extern "C" int ra_gemm_wide_partial(const void* A, const void* W, float* P, long
            "gemm_wide: operands must be 16-byte aligned");
   int waves, S, kps;
   bool partial;
-  gw_split(WEPI_PLAIN, N, K, &waves, &S, &kps, &partial, true);
+  gw_split(WEPI_PLAIN, M, N, K, &waves, &S, &kps, &partial, true);
   RA_CHECK(P && p_floats >= (long)S * M * N, "gemm_wide: %d ranges of [%d, %d] need %ld floats, got %ld", S, M, N,
            (long)S * M * N, p_floats);
   const WideNorm nf = {};
 #define RA_GWP(MT, WV)                                                                                  \
   gemm_wide_kernel<MT, WV, WEPI_PARTIAL, float><<<dim3((N + WV * 16 - 1) / (WV * 16), S), WV * RA_WAVE, 0, stream>>>( \
       (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, P, N, M, N, K, kps, nf)
-#define RA_GWPM(MT)              \
-  do {                           \
-    if (waves == 6) RA_GWP(MT, 6); \
-    else RA_GWP(MT, 8);          \
-  } while (0)
+#define RA_GWPM(MT) RA_GWP(MT, 8)          /* a product cut into K ranges has workgroups of 8 waves */
   if (M <= 16) RA_GWPM(1);
   else if (M <= 32) RA_GWPM(2);
   else if (M <= 48) RA_GWPM(3);

@@ -598,7 +598,7 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
     width of 4096); a gated product wide enough to fill the chip goes to the kernel whose waves
     share the activations at every row count, and adds them up itself."""
     torch.manual_seed(M)
-    N, K, J, eps = 4096, 256, 9216, 1e-6
+    N, K, J, eps = 4096, 256, 12288, 1e-6      # 24576 gated features: 256 workgroups of 96, one a CU
     a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w1 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
     stream = torch.randn(M, N, device=DEV) * 3
