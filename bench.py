@@ -222,7 +222,7 @@ def main() -> int:
         return 2
     max_new = prompt_steps + args.warmup + args.steps + 16
     blocks_per_req = -(-(args.prompt_len + max_new + 32) // block) + 1
-    num_blocks = max_batch * blocks_per_req + 8
+    num_blocks = max(max_batch * blocks_per_req, -(-(args.prefill_tokens + 16) // block)) + 8
     log(f"building {raw['num_hidden_layers']} layers of the {shape_name} shape in {args.dtype}, random weights ...")
     t0 = time.perf_counter()
     engine = LLMEngine(config=cfg, seed=args.seed, dtype=args.dtype, block_size=block, num_blocks=num_blocks,
