@@ -161,6 +161,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     if "--" in argv:
         cut = argv.index("--")
         argv, prompt = argv[:cut], argv[cut + 1:]
+    if argv and argv[0] == "bench":
+        # everything behind the verb is bench.py's, options first or not
+        args = argparse.Namespace(verb="bench", rest=argv[1:] + (["--"] + prompt if prompt else []), fn=cmd_bench)
+        return args.fn(args)
     args, extra = ap.parse_known_args(argv)
     if extra:
         if args.verb not in ("run", "generate") or any(w.startswith("-") and not w.lstrip("-").isdigit() for w in extra):

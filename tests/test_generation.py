@@ -137,3 +137,11 @@ def test_command_line_backend_option():
     with pytest.raises(SystemExit):
         cli.main(["run", "m", "--backend", "cuda"])
     assert cli._backend("auto") == "auto" and cli._backend("hip") == "hip"
+
+
+def test_command_line_bench_passes_options_on():
+    """`reinfer bench --gpus 2` hands everything behind the verb to bench.py, options first or not:
+    bench.py says that it runs on one GPU and the exit status is its 2."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "reinfer"), "bench", "--gpus", "2"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 2 and "one GPU" in r.stdout
