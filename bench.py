@@ -216,10 +216,14 @@ def main() -> int:
     # a request decodes while later prompts are still being prefilled: one step a portion of a prompt
     budget = max(2048, args.prefill_tokens)
     prompt_steps = max_batch * -(-args.prompt_len // budget)
-    if args.prompt_len + prompt_steps + args.warmup + args.steps + 16 > ctx_len:
-        print(f"bench.py: {max_batch} prompts of {args.prompt_len} tokens and {args.warmup + args.steps} decode steps "
-              f"do not fit a context of {ctx_len}", file=sys.stderr)
-        return 2
+    need_ctx = max(args.prompt_len + prompt_steps + args.warmup + args.steps + 16, args.prefill_tokens + 8)
+    if need_ctx > ctx_len:
+        # exactly the steps asked for are timed: a run that outgrows the shape's context gets a longer one
+        ctx_len = -(-need_ctx // 1024) * 1024
+        raw["max_position_embeddings"] = ctx_len
+        cfg = config_from_dict(raw)
+        log(f"{max_batch} prompts of {args.prompt_len} tokens, {args.warmup + args.steps} decode steps and a prefill of "
+            f"{args.prefill_tokens} need a context of {ctx_len}")
     max_new = prompt_steps + args.warmup + args.steps + 16
     blocks_per_req = -(-(args.prompt_len + max_new + 32) // block) + 1
     num_blocks = max(max_batch * blocks_per_req, -(-(args.prefill_tokens + 16) // block)) + 8

@@ -164,8 +164,10 @@ class DecodeGraphs:
         entries are padding; both are overwritten by the next replay of this bucket."""
         r = self.runner
         B = _batch_bucket(len(entries))
-        ctx_cap = max(256, _bucket(longest))
-        ctx_cap = min(ctx_cap, max(256, _bucket(r.max_model_len)))
+        # context buckets are powers of two from 256, and never more than the block tables hold (a
+        # context limit that is no power of two, or below 256, is its own last bucket)
+        table_room = max(1, -(-r.max_model_len // r.block_size)) * r.block_size
+        ctx_cap = min(max(256, _bucket(longest)), table_room)
         key = (B, ctx_cap)
         cs = self.steps.get(key)
         if cs is None:

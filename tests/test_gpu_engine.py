@@ -294,3 +294,17 @@ def test_thousands_of_tokens_of_context(tmp_path, which, dtype):
     got = run_plan(runner, {"r": toks}, plan)["r"]
     assert rel_err(got, ref) < TOL[dtype]
     assert rel_err(got[-64:], ref[-64:]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("limit,n", [(300, 299), (100, 99)])
+def test_context_limit_that_is_no_power_of_two(folders, plain_cache, limit, n):
+    """Captured decode steps pad the context to buckets (powers of two from 256); the last bucket is the
+    context limit itself, which the block tables are made for: 300 (contexts above 256 once asked for a
+    bucket of 512 that the tables did not hold) and 100 (below the smallest bucket)."""
+    which, dtype = "B", "bfloat16"
+    runner = runner_for(folders, which, dtype, max_tokens=320, max_model_len=limit)
+    toks = random_tokens(n, vocab(which), 88)
+    first = n - 60
+    got = run_plan(runner, {"r": toks}, [[("r", first)]] + [[("r", 1)]] * 60)["r"]
+    assert runner.graphs is not None and runner.graphs.replays >= 60
+    assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype]
