@@ -25,7 +25,8 @@ def draw_config(rng):
            "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 256]),
            "intermediate_size": rng.choice([88, 176, 456, 1000, 1368]), "vocab_size": rng.choice([333, 1003, 5001]),
            "rope_theta": rng.choice([10000.0, 1e6, 5e4]), "rms_norm_eps": rng.choice([1e-6, 1e-5, 3e-4]),
-           "tie_word_embeddings": rng.random() < 0.5, "max_position_embeddings": 1024, "attention_bias": False,
+           "tie_word_embeddings": rng.random() < 0.5, "max_position_embeddings": rng.choice([521, 600, 777, 1000, 1024]),
+           "attention_bias": False,
            "hidden_act": "silu", "rope_scaling": None, "sliding_window": None, "use_sliding_window": False}
     if rng.random() < 0.4:
         raw.update(sliding_window=rng.choice([5, 16, 21, 64, 100]), use_sliding_window=True,
