@@ -54,8 +54,10 @@ class RMSNorm:
         ops = kernels.current()
         parts = getattr(ops, "skinny_row_parts", None)
         T = resid.shape[0]
+        # the product behind this norm reads rows of this width as 16-byte pieces: a width that is no
+        # multiple of 8 goes through the norm kernel and the plain product
         if parts is None or self.dtype != torch.bfloat16 or T > getattr(ops, "NORM_ON_PRODUCTS_ROWS", 0) \
-                or resid.shape[1] != self.size:
+                or resid.shape[1] != self.size or self.size % 8 != 0:
             return None
         return NormTarget(self,
                           torch.empty((T, self.size), dtype=torch.bfloat16, device=resid.device),

@@ -83,3 +83,36 @@ def test_random_configurations_and_plans(tmp_path, seed, dtype):
         for r, toks in seqs.items():
             err = rel_err(got[r], plain.forward(rawr, weights, toks).float())
             assert err < TOL[dtype], (seed, ci, r, raw, plan[:8])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [
+    dict(hidden_size=132, intermediate_size=260, head_dim=16, num_attention_heads=9, num_key_value_heads=9, vocab_size=1001),
+    dict(hidden_size=100, intermediate_size=90, head_dim=32, num_attention_heads=6, num_key_value_heads=3, vocab_size=257),
+    dict(hidden_size=200, intermediate_size=4, head_dim=32, num_attention_heads=2, num_key_value_heads=2, vocab_size=2),
+])
+def test_sizes_that_the_matrix_core_kernels_do_not_take(tmp_path, sizes, dtype):
+    """Widths that are no multiple of 8 (rows are not whole 16-byte pieces), a feed-forward of 4, a
+    vocabulary of 2: what the weight-streaming kernels refuse goes to the plain kernels, at every row
+    count, with no norm riding on a product that cannot carry it."""
+    raw = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": sizes["vocab_size"] % 2 == 1, "max_position_embeddings": 300, **sizes}
+    folder = str(tmp_path / "m")
+    write_model_folder(config_from_dict(raw), 5, folder, dtype=dtype)
+    rawr, weights = read_folder(folder)
+    seqs = {r: random_tokens(n, raw["vocab_size"], 9 + i) for i, (r, n) in enumerate((("a", 150), ("b", 70), ("c", 9)))}
+    runner = ModelRunner.from_folder(folder, dtype=dtype, device="cuda:0", max_tokens=320)
+    plan = [[("a", 100), ("b", 2)], [("a", 1), ("b", 66), ("c", 9)], [("a", 49), ("b", 1)], [("b", 1)]]
+    got = run_plan(runner, seqs, plan)
+    for r, toks in seqs.items():
+        assert rel_err(got[r], plain.forward(rawr, weights, toks).float()) < TOL[dtype], r
+
+
+def test_head_size_that_is_no_multiple_of_16_is_refused(tmp_path):
+    raw = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 1, "hidden_size": 64, "intermediate_size": 96,
+           "head_dim": 24, "num_attention_heads": 4, "num_key_value_heads": 2, "vocab_size": 100,
+           "max_position_embeddings": 64}
+    folder = str(tmp_path / "m")
+    write_model_folder(config_from_dict(raw), 0, folder, dtype="bfloat16")
+    with pytest.raises(ValueError, match="steps of 16"):
+        ModelRunner.from_folder(folder, dtype="bfloat16", device="cuda:0", max_tokens=64)
