@@ -145,3 +145,37 @@ def test_command_line_bench_passes_options_on():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "reinfer"), "bench", "--gpus", "2"],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 2 and "one GPU" in r.stdout
+
+
+@pytest.mark.gpu
+def test_many_requests_with_mixed_sampling_do_not_depend_on_the_batch(tmp_path):
+    """Forty requests of many lengths and caps, greedy beside temperature, top-k / top-p, min-p with a
+    repeat penalty and stop ids: run together (portions of 96 tokens beside up to 32 decoding requests),
+    each alone, and together in a pool so small that requests are preempted and recomputed. In 32-bit
+    every kernel sums in a fixed order, so the tokens and the finish reasons are the same."""
+    import random
+    folder = make_folder(tmp_path, "C", "float32")
+    raw, _ = read_folder(folder)
+    V = raw["vocab_size"]
+    rng = random.Random(1)
+    prompts, params = [], []
+    for i in range(40):
+        prompts.append(random_tokens(rng.choice([1, 2, 5, 17, 33, 64, 65, 100, 130]), V, 1000 + i))
+        cap = rng.choice([1, 2, 7, 30, 60])
+        params.append([SamplingParams(temperature=0.0, max_tokens=cap),
+                       SamplingParams(temperature=0.8, seed=50 + i, max_tokens=cap),
+                       SamplingParams(temperature=0.9, seed=50 + i, top_k=20, top_p=0.9, max_tokens=cap),
+                       SamplingParams(temperature=0.7, seed=50 + i, min_p=0.05, repeat_penalty=1.2, max_tokens=cap,
+                                      stop_token_ids=[3, 4, 5])][i % 4])
+    limits = dict(max_num_batched_tokens=96, max_model_len=250)
+    eng = engine_for(folder, "cuda:0", num_blocks=200, max_num_seqs=32, **limits)
+    together = eng.generate(prompts, params)
+    assert eng.cache_stats()["blocks_free"] == eng.cache_stats()["blocks_total"]
+    one = engine_for(folder, "cuda:0", num_blocks=32, max_num_seqs=2, **limits)
+    for i, (p, sp) in enumerate(zip(prompts, params)):
+        alone = one.generate([p], sp)[0]
+        assert (alone.token_ids, alone.finish_reason) == (together[i].token_ids, together[i].finish_reason), i
+    small = engine_for(folder, "cuda:0", num_blocks=40, max_num_seqs=32, admission="blocks", **limits)
+    again = small.generate(prompts, params)
+    assert small.cache_stats()["preemptions"] > 0
+    assert [o.token_ids for o in again] == [o.token_ids for o in together]
