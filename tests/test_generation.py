@@ -179,3 +179,36 @@ def test_many_requests_with_mixed_sampling_do_not_depend_on_the_batch(tmp_path):
     again = small.generate(prompts, params)
     assert small.cache_stats()["preemptions"] > 0
     assert [o.token_ids for o in again] == [o.token_ids for o in together]
+
+
+@pytest.mark.gpu
+def test_aborts_and_arrivals_between_captured_decode_steps(tmp_path):
+    """Requests are aborted and others arrive while the rest decode from captured steps: the rows of
+    a captured step change hands (another request, another block table), a request id comes back from
+    its start, every block returns, and in 32-bit each finished request has the tokens it has alone."""
+    folder = make_folder(tmp_path, "B", "float32")
+    raw, _ = read_folder(folder)
+    V = raw["vocab_size"]
+    P = {k: random_tokens(n, V, 10 + i) for i, (k, n) in enumerate((("a", 20), ("b", 35), ("c", 9), ("d", 50), ("e", 28), ("f", 3)))}
+    sp = SamplingParams(temperature=0.0, max_tokens=40)
+    one = engine_for(folder, "cuda:0", num_blocks=64, max_num_seqs=2)
+    alone = {k: one.generate([p], sp)[0].token_ids for k, p in P.items()}
+    eng = engine_for(folder, "cuda:0", num_blocks=64, max_num_seqs=8)
+    for k in "abcd":
+        eng.add_request(P[k], sp, rid=k)
+    outs, step = {}, 0
+    while eng.has_unfinished():
+        for o in eng.step():
+            outs[o.rid] = o
+        step += 1
+        if step == 8:
+            assert eng.abort("b") and not eng.abort("b")
+            eng.add_request(P["e"], sp, rid="e")
+        if step == 15:
+            assert eng.abort("a")
+            eng.add_request(P["f"], sp, rid="f")
+            eng.add_request(P["b"], sp, rid="b")
+    assert sorted(outs) == ["b", "c", "d", "e", "f"]
+    assert {k: outs[k].token_ids for k in outs} == {k: alone[k] for k in outs}
+    assert eng.runner.graphs is not None and eng.runner.graphs.replays > 30
+    assert eng.cache_stats()["blocks_free"] == eng.cache_stats()["blocks_total"]
