@@ -91,3 +91,34 @@ def test_trace_run_orders_ids_and_idle_requests(tmp_path, which, dtype):
             continue
         got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(ref.shape[0], V))
         assert rel_err(got, ref) < TOL[dtype], s["step"]
+
+
+def test_trace_run_step_by_step_over_a_pipe(tmp_path):
+    """The caller writes one step, waits for ``done <step>``, then writes the next: every answer comes
+    without further input, the step's file is whole when the answer is printed, and the end of the
+    input ends the program with status 0."""
+    folder = make_folder(tmp_path, "A", "bfloat16")
+    raw, weights = read_folder(folder)
+    toks = random_tokens(24, raw["vocab_size"], 5)
+    ref = plain.forward(raw, weights, toks).float()
+    out = tmp_path / "out"
+    proc = subprocess.Popen(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "bfloat16",
+         "--out", str(out), "--max-tokens", "64"],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
+    try:
+        fed = 0
+        for step in range(13):
+            n = 12 if step == 0 else 1
+            rec = {"step": step, "entries": [{"id": "a", "tokens": toks[fed:fed + n], "want": [n - 1]}], "end": []}
+            proc.stdin.write(json.dumps(rec) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {step}"
+            fed += n
+            got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(1, -1))
+            assert rel_err(got, ref[fed - 1:fed]) < TOL["bfloat16"]
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
