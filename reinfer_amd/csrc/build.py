@@ -78,7 +78,11 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError("hipcc not found: the gfx950 kernel library cannot be built "
                            "(set HIPCC or put /opt/rocm/bin on PATH)")
     out_dir = _writable_dir()
-    obj_dir = os.path.join(out_dir, "_build")
+    stamp_dir = os.path.join(out_dir, "_build")
+    # objects in a folder of this process: two programs that find nothing built at the same moment
+    # (two replays started side by side in a fresh tree) each build whole objects and publish the
+    # library with one rename
+    obj_dir = os.path.join(stamp_dir, f"obj_{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
     env = dict(os.environ)
@@ -112,8 +116,9 @@ def build(verbose: bool = True) -> str:
     if r.returncode != 0:
         raise RuntimeError(f"hipcc link failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
-    with open(os.path.join(obj_dir, "source.sha256"), "w") as f:
+    with open(os.path.join(stamp_dir, "source.sha256"), "w") as f:
         f.write(source_hash())
+    shutil.rmtree(obj_dir, ignore_errors=True)
     if verbose:
         _say(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
