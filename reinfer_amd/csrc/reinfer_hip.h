@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 14
+#define RA_ABI_VERSION 15
 
 #ifdef __cplusplus
 extern "C" {
@@ -118,6 +118,17 @@ int ra_sample_slices(int vocab);
 int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,
               const long long* seeds, const int* positions, float* scratch_val, int* scratch_idx,
               int* tokens, hipStream_t stream);
+
+// ra_sample for callers that cannot allocate device memory (code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The slice
+// winners go to an array that the library holds on every GPU it runs on (512 KiB, until the process
+// ends) instead of caller buffers; inputs and `tokens` are still the caller's. It calls no hipMalloc,
+// hipFree or allocating routine; n_rows * ra_sample_slices(vocab) may be at most
+// ra_sample_static_max_pairs() (65536), more is refused with a message. All calls on one GPU share that
+// GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+long ra_sample_static_max_pairs(void);
+int ra_sample_static(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,
+                     const long long* seeds, const int* positions, int* tokens, hipStream_t stream);
 
 // Logit bias, penalties and filters on rows of float logits, in place, before ra_sample. `rows`
 // holds one record of 12 x 4 bytes per row: float temperature, top_p, min_p, repeat_penalty,

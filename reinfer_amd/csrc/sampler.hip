@@ -12,6 +12,7 @@
 // The reference's sampler is one 256-thread workgroup
 // (sampler_kernel.cu:157); here stage 1 scans slices of the row in parallel
 // and stage 2 merges the slice winners in a fixed order.
+#include <mutex>
 #include "common.h"
 #include "reinfer_hip.h"
 
@@ -120,6 +121,68 @@ extern "C" int ra_sample(const float* logits, int n_rows, int vocab, int row_str
   RA_LAUNCH_CHECK("sample stage 1");
   sample_stage2<<<n_rows, SAMPLE_THREADS, 0, stream>>>(scratch_val, scratch_idx, n_slices, tokens);
   RA_LAUNCH_CHECK("sample stage 2");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The same two stages for callers that cannot allocate: the slice winners go
+// to a file-scope array of device memory instead of buffers the caller brings.
+// Each GPU holds its own copy of the array, at its own address, until the
+// process ends (SAMPLE_STATIC_PAIRS * 8 bytes = 512 KiB). In host code the
+// array's name is only a handle for hipGetSymbolAddress: the address it
+// yields, looked up once per device with that device current, is what the
+// kernels get. Stage 1 writes every pair that stage 2 reads, so nothing has to
+// be cleared between calls; what an earlier call left beyond that is never read.
+// ---------------------------------------------------------------------------
+#define SAMPLE_STATIC_PAIRS 65536            // (row, slice) pairs a call may need
+#define SAMPLE_STATIC_DEVICES 64
+
+static __device__ __align__(256) unsigned char scratch[SAMPLE_STATIC_PAIRS * (sizeof(float) + sizeof(int))];
+
+static void* scratch_of_device[SAMPLE_STATIC_DEVICES];     // device address of `scratch`, per GPU
+static std::mutex scratch_lock;
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  RA_CHECK(e == hipSuccess, "sample_static: no current device: %s", hipGetErrorString(e));
+  RA_CHECK(dev >= 0 && dev < SAMPLE_STATIC_DEVICES, "sample_static: device %d (at most %d are known)", dev,
+           SAMPLE_STATIC_DEVICES);
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (scratch_of_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    RA_CHECK(e == hipSuccess && p != nullptr, "sample_static: the scratch array has no address on device %d: %s", dev,
+             hipGetErrorString(e));
+    scratch_of_device[dev] = p;
+  }
+  *out = scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" long ra_sample_static_max_pairs(void) { return SAMPLE_STATIC_PAIRS; }
+
+extern "C" int ra_sample_static(const float* logits, int n_rows, int vocab, int row_stride,
+                                const float* temperature, const long long* seeds, const int* positions,
+                                int* tokens, hipStream_t stream) {
+  RA_CHECK(n_rows > 0 && vocab > 0, "sample_static: empty input (%d rows, vocabulary %d)", n_rows, vocab);
+  RA_CHECK(row_stride >= vocab, "sample_static: row stride %d below the vocabulary %d", row_stride, vocab);
+  RA_CHECK(n_rows <= 65535, "sample_static: %d rows in one launch (max 65535)", n_rows);
+  const int n_slices = ra_sample_slices(vocab);
+  RA_CHECK((long)n_rows * n_slices <= SAMPLE_STATIC_PAIRS,
+           "sample_static: %d rows of %d slices need %ld pairs of scratch, the array holds %d "
+           "(use ra_sample with buffers of your own)",
+           n_rows, n_slices, (long)n_rows * n_slices, SAMPLE_STATIC_PAIRS);
+  void* base = nullptr;
+  if (static_scratch(&base) != 0) return 1;
+  float* part_val = (float*)base;
+  int* part_idx = (int*)((unsigned char*)base + SAMPLE_STATIC_PAIRS * sizeof(float));
+  dim3 grid(n_slices, n_rows);
+  sample_stage1<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, vocab, row_stride, temperature, seeds,
+                                                     positions, part_val, part_idx, n_slices);
+  RA_LAUNCH_CHECK("sample_static stage 1");
+  sample_stage2<<<n_rows, SAMPLE_THREADS, 0, stream>>>(part_val, part_idx, n_slices, tokens);
+  RA_LAUNCH_CHECK("sample_static stage 2");
   return 0;
 }
 

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 
 class KernelLibraryError(RuntimeError):
@@ -44,6 +44,7 @@ _SIGNATURES = {
     "ra_gemm_skinny_normed": [P, P, P, P, I, I, I, I, I, I, I, P, I, F, I, P, I, P, I, P, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],
+    "ra_sample_static": [P, I, I, I, P, P, P, P, P],
     "ra_filter_logits": [P, I, I, I, P, P, P],
     "ra_stream_read": [P, c_long, P, P],
     "ra_mfma_loop": [I, I, I, P, P, P],
@@ -78,6 +79,8 @@ def load() -> ctypes.CDLL:
         for name in ("ra_attention_prefill_tile", "ra_attention_prefill_columns", "ra_attention_prefill_groups"):
             getattr(lib, name).restype = c_int
             getattr(lib, name).argtypes = [c_int, c_int, c_int]
+        lib.ra_sample_static_max_pairs.restype = c_long
+        lib.ra_sample_static_max_pairs.argtypes = []
         lib.ra_gemm_skinny_max_rows.restype = c_int
         lib.ra_gemm_skinny_max_rows.argtypes = []
         lib.ra_gemm_skinny_row_parts.restype = c_int
