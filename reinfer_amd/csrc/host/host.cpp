@@ -691,7 +691,14 @@ struct Scheduler {
     }
     req->state = FINISHED;
     req->finish_reason = py::str("abort");
+    forget(req);
     return true;
+  }
+  // A finished request leaves the table: whoever holds the Request object keeps it alive, the
+  // scheduler keeps nothing of it (a long-running engine's memory does not grow with requests served).
+  void forget(const RequestP& req) {
+    auto it = requests.find(req->rid);
+    if (it != requests.end() && it->second == req) requests.erase(it);
   }
   bool has_work() const { return !waiting.empty() || !running.empty(); }
 
@@ -787,6 +794,7 @@ struct Scheduler {
         lone->state = FINISHED;
         lone->finish_reason = py::str("cache");
         ++c_finished;
+        forget(lone);
         plan.finished.push_back(lone);
         break;
       }
@@ -829,15 +837,40 @@ struct Scheduler {
       return 0;
     };
 
-    // 2. prompt portions of running requests, oldest first
-    for (auto& r : by_arrival) {
-      if (r->decoding()) continue;
-      if (left <= 0) break;
-      const int n = fit(r, r->num_computed, std::min({r->remaining(), max_chunk, left}), true, 0);
-      if (n > 0) {
-        plan.portions.push_back(Portion{r, r->num_computed, n});
-        left -= n;
+    // 2. prompt portions of running requests, oldest first. If nothing at all can be placed (every
+    // running request is in the middle of its prompt and the pool is full, so that step 1 had nobody to
+    // make room for), the newest request that was not preempted before goes back to the queue and its
+    // blocks serve the others; a lone request that cannot get a block ends with reason `cache`.
+    while (true) {
+      for (auto& r : by_arrival) {
+        if (r->decoding()) continue;
+        if (left <= 0) break;
+        const int n = fit(r, r->num_computed, std::min({r->remaining(), max_chunk, left}), true, 0);
+        if (n > 0) {
+          plan.portions.push_back(Portion{r, r->num_computed, n});
+          left -= n;
+        }
       }
+      if (!plan.portions.empty() || running.empty() || left <= 0) break;
+      if (running.size() == 1) {
+        // it may still be admitted again below if it was the pool's only holder: only a request that
+        // holds the whole pool and still needs more ends here
+        auto lone = running[0];
+        running.clear();
+        manager->free(lone->rid);
+        lone->state = FINISHED;
+        lone->finish_reason = py::str("cache");
+        ++c_finished;
+        forget(lone);
+        plan.finished.push_back(lone);
+        break;
+      }
+      RequestP victim = running[0];
+      for (auto& r : running)
+        if (std::make_pair(r->resumed, -r->arrival) < std::make_pair(victim->resumed, -victim->arrival)) victim = r;
+      preempt(victim, plan);
+      by_arrival.erase(std::find(by_arrival.begin(), by_arrival.end(), victim));
+      read_free();
     }
 
     // 3. admissions: resumed first (they sit at the head), then arrival order
@@ -927,6 +960,7 @@ struct Scheduler {
         manager->free(r->rid);
         ++c_finished;
         observe_output((long)r->output.size());
+        forget(r);
         done.push_back(r);
       }
     }
