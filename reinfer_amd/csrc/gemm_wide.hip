@@ -310,19 +310,21 @@ static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int*
 
 // 1 where this kernel beats ra_gemm_skinny (measured on MI355X at 4 to 64 rows): from 17 rows on,
 // except a small product whose K has to be cut (4096 x 4096: the second launch costs more than the
-// shared activations save); below that for the gated product of a wide feed-forward.
+// shared activations save); from 9 rows for the gated product of a wide feed-forward.
 extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
   if (M < 1 || M > 64) return 0;
   int waves, S, kps;
   gw_split(epilogue, M, N, K, &waves, &S, &kps);
-  // below 17 rows the gated product of a wide feed-forward: one K range, enough workgroups to fill the
-  // chip (measured at 4 to 16 rows, 24576 x 4096: 37 us against 39 to 42) and to fill whole rounds of it
+  // from 9 to 16 rows the gated product of a wide feed-forward (up to 8 rows the other kernel, whose
+  // workgroups stay and keep two runs a wave in flight, is ahead: 24576 x 4096 36 us against 37, 51200 x
+  // 5120 91 to 97 against 101 to 103): one K range, enough workgroups to fill the
+  // chip (measured at 16 rows, 24576 x 4096: 37 us against 41) and to fill whole rounds of it
   // (400 workgroups would leave a third of the CUs with half the work: the other kernel's many small
   // ones are then faster); and from 9 rows a plain product over a vocabulary (151936 features at 16 rows,
   // K = 2560 / 4096 / 5120: 148 / 237 / 280 us against 170 / 239 / 327)
   const int cb = (N + waves * 16 - 1) / (waves * 16);
   if (M < 17) {
-    if (epilogue == WEPI_SILU_PAIRS) return (S == 1 && cb >= 192 && cb * 10 >= ((cb + 255) / 256) * 256 * 8) ? 1 : 0;
+    if (epilogue == WEPI_SILU_PAIRS) return (M > 8 && S == 1 && cb >= 192 && cb * 10 >= ((cb + 255) / 256) * 256 * 8) ? 1 : 0;
     return (epilogue == WEPI_PLAIN && M > 8 && S == 1 && cb >= 768) ? 1 : 0;
   }
   return (S == 1 || (long)N * K > 4096L * 4096L) ? 1 : 0;
