@@ -16,11 +16,14 @@
 // 4g + s of the first 16 keys for s < 4, of the second 16 for s >= 4, for both
 // operands alike).
 //
-// The grid is a fixed number of workgroups, as many as the chip holds at once; the
-// (token, chunk, KV head) items are numbered on the device from the tokens'
-// positions and workgroup w takes items w, w + grid, ...: launching one
-// workgroup an item costs 13 to 20 ns each (a step of 64 requests has ten
-// thousand) and leaves the last round of workgroups half empty.
+// The grid is a fixed number of workgroups, as many as the chip holds at once; every
+// token has max_chunks items a KV head (those past its own number of chunks are
+// empty) and workgroup w takes items w, w + grid, ...: launching one workgroup an
+// item costs 13 to 20 ns each (a step of 64 requests has ten thousand) and leaves
+// the last round of workgroups half empty. An item's token and chunk follow from
+// its number, not from a table built from all tokens' positions first: in a
+// launch that lasts some ten microseconds every trip to memory that another
+// waits for shows (here: arguments, position and request, block ids, keys).
 //
 // Chunks of one (token, head) are merged by a second small kernel, always in
 // chunk order. (Merging in the last workgroup to arrive needs device-wide
@@ -37,7 +40,6 @@
 
 #define FD_THREADS 256
 #define FD_WAVES 4
-#define FD_MAX_TOKENS 1024      // tokens of one launch; the entry point cuts longer lists
 
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -76,53 +78,24 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
   extern __shared__ float lds[];       // [waves][G][d] outputs, then [waves][G][2] maximum and sum
 
-  __shared__ int first_item[FD_MAX_TOKENS + 1];   // chunks of the tokens before token i
-
   const int tid = threadIdx.x;
   const int lane = tid & (RA_WAVE - 1), wave = tid / RA_WAVE;
   const int r = lane & 15, g = lane >> 4;
 
-  // every workgroup numbers the items alike: chunks of each token, then a running sum
-  for (int i = tid; i < n_tokens; i += FD_THREADS) {
-    const int pi = positions[token_list ? token_list[i] : t_base + i];
-    const int loi = (window > 0 && pi - window + 1 > 0) ? pi - window + 1 : 0;
-    first_item[i + 1] = fd_cut(pi, loi, chunk_shift, max_chunks).n;
-  }
-  if (tid == 0) first_item[0] = 0;
-  __syncthreads();
-  if (wave == 0) {
-    const int per = (n_tokens + RA_WAVE - 1) / RA_WAVE;
-    const int b = lane * per;
-    int sum = 0;
-    for (int j = 0; j < per; ++j)
-      if (b + j < n_tokens) sum += first_item[b + j + 1];
-    int incl = sum;
-#pragma unroll
-    for (int o = 1; o < RA_WAVE; o <<= 1) {
-      const int up = __shfl_up(incl, o, RA_WAVE);
-      if (lane >= o) incl += up;
-    }
-    int run = incl - sum;
-    for (int j = 0; j < per; ++j)
-      if (b + j < n_tokens) {
-        run += first_item[b + j + 1];
-        first_item[b + j + 1] = run;
-      }
-  }
-  __syncthreads();
-  const int n_items = first_item[n_tokens] * Hkv;
-
-  int li = 0;                                     // items of a workgroup ascend: the token only moves forward
+  // Item i is (token i / (max_chunks * Hkv), chunk (i / Hkv) % max_chunks, KV head i % Hkv): known from
+  // the item's number alone, so the first trip to memory is already the token's own position and
+  // request. A token whose keys make fewer chunks leaves its last items empty (they end here).
+  const int n_items = n_tokens * max_chunks * Hkv;
   for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
     const int slot = item / Hkv, kvh = item % Hkv;  // KV heads of one (token, chunk) are neighbours in memory
-    while (first_item[li + 1] <= slot) ++li;
+    const int li = slot / max_chunks, ci = slot % max_chunks;
     const int t = token_list ? token_list[li] : t_base + li;
     const int p = positions[t];
+    const int seq = seq_of_token[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const FdCut cut = fd_cut(p, lo, chunk_shift, max_chunks);
-    const int ci = slot - first_item[li];
     const int n_chunks = cut.n;
-    const int seq = seq_of_token[t];
+    if (ci >= n_chunks) continue;
     const int* table = block_tables + (size_t)seq * max_blocks;
     const int Hq = Hkv * G;
 
@@ -293,22 +266,72 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
   }
 }
 
-// Merge of the chunks of one (token, head), one wave each: lane c weighs chunk c
-// (all maxima and sums are read at once), then the lanes share the d outputs.
+// Merge of the chunks of one (token, head), one wave each: lane c weighs chunk c, then the lanes share
+// the d outputs. With up to FDM_AHEAD chunks a token everything the wave may need (the maxima and sums
+// and the partial outputs of all max_chunks rows) is asked for at once, beside the token's position,
+// before the number of chunks is known: rows past it hold whatever was there and are left out by
+// selection, never by a factor of zero. That is one trip to memory instead of three in a row.
+#define FDM_AHEAD 16
+// AHEAD = outputs a lane (1, 2 or 4: head sizes up to 64, 128, 256) of the form that asks ahead; 0: the general form
+template <int AHEAD>
 __global__ void __launch_bounds__(RA_WAVE)
 flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                           bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
                           const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk_shift,
                           int max_chunks, int t_base) {
   const int head = blockIdx.x, li = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int kvh = head / G, h = head % G;
+  const size_t base = ((size_t)li * Hkv + kvh) * max_chunks * G + h;    // row of chunk 0; chunks are G rows apart
   const int t = token_list ? token_list[li] : t_base + li;
+  if (AHEAD) {
+    // max_chunks <= FDM_AHEAD, d <= 64 * AHEAD
+    constexpr int EPL = AHEAD > 0 ? AHEAD : 1;
+    float v[FDM_AHEAD][EPL];
+    const int cl = lane < max_chunks ? lane : max_chunks - 1;
+    const float mc_raw = part_ml[(base + (size_t)cl * G) * 2];
+    const float lc_raw = part_ml[(base + (size_t)cl * G) * 2 + 1];
+#pragma unroll
+    for (int c = 0; c < FDM_AHEAD; ++c) {
+      const float* po = part_o + (base + (size_t)(c < max_chunks ? c : max_chunks - 1) * G) * d;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + i * RA_WAVE;
+        v[c][i] = po[e < d ? e : d - 1];
+      }
+    }
+    const int p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks).n;
+    if (n_chunks == 1) return;                           // written by the first kernel
+    const bool mine = lane < n_chunks;
+    const float mc = mine ? mc_raw : -INFINITY, lc = mine ? lc_raw : 0.f;
+    const float mt = wave_max(mc);                       // finite: every chunk saw at least one key
+    const float w = mine ? fd_exp2(mc - mt) : 0.f;
+    const float lt = wave_sum(lc * w);
+    float acc[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < FDM_AHEAD; ++c) {
+      const float wc = __shfl(w, c, RA_WAVE);
+      if (c < n_chunks) {                                // uniform; chunk order
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) acc[i] += v[c][i] * wc;
+      }
+    }
+    const float inv = 1.f / lt;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + i * RA_WAVE;
+      if (e < d) out[(size_t)t * out_stride + (size_t)head * d + e] = from_f32<bf16_t>(acc[i] * inv);
+    }
+    return;
+  }
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks).n;
   if (n_chunks == 1) return;                           // written by the first kernel
-  const int lane = threadIdx.x;
-  const int kvh = head / G, h = head % G;
-  const size_t base = ((size_t)li * Hkv + kvh) * max_chunks * G + h;    // row of chunk 0; chunks are G rows apart
   float acc[4] = {0.f, 0.f, 0.f, 0.f};                 // d <= 256: up to 4 outputs a lane
   float mt = -INFINITY, lt = 0.f;
   for (int c0 = 0; c0 < n_chunks; c0 += RA_WAVE) {
@@ -417,37 +440,37 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
   RA_CHECK(lds <= 64 * 1024, "attention_decode: %d heads of %d per KV head need too much LDS", G, d);
   const int slots = fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, lds);
   RA_CHECK(slots > 0, "attention_decode: cannot size the grid (%s)", hipGetErrorString(hipGetLastError()));
-  // lists longer than the kernel's item table go in slices, each with its part of the partial buffers
-  for (int base = 0; base < n_tokens; base += FD_MAX_TOKENS) {
-    const int n = n_tokens - base < FD_MAX_TOKENS ? n_tokens - base : FD_MAX_TOKENS;
-    const int* list = token_list ? token_list + base : nullptr;
-    const size_t rows = (size_t)base * Hkv * max_chunks * G;
-    float* po = part_o ? part_o + rows * d : nullptr;
-    float* pm = part_ml ? part_ml + rows * 2 : nullptr;
-    const long items_max = (long)n * Hkv * max_chunks;
-    const int grid = (int)(items_max < slots ? items_max : slots);
+  const long items_max = (long)n_tokens * Hkv * max_chunks;
+  RA_CHECK(items_max < (1L << 30), "attention_decode: %ld work items in one launch", items_max);
+  const int grid = (int)(items_max < slots ? items_max : slots);
 #define RA_FD_GO(DM, EX)                                                                              \
   flash_decode_kernel<DM, EX><<<grid, FD_THREADS, lds, stream>>>(                                     \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
-      (const bf16_t*)vcache, block_tables, max_blocks, list, seq_of_token, positions, block_size,     \
-      Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n, base, po, pm)
+      (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size, \
+      Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml)
 #define RA_FD(DM)                                                                                     \
   do {                                                                                                \
     if (d == DM) RA_FD_GO(DM, true);                                                                  \
     else RA_FD_GO(DM, false);                                                                         \
   } while (0)
-    if (d <= 64) RA_FD(64);
-    else if (d <= 128) RA_FD(128);
-    else RA_FD(256);
+  if (d <= 64) RA_FD(64);
+  else if (d <= 128) RA_FD(128);
+  else RA_FD(256);
 #undef RA_FD_GO
 #undef RA_FD
-    RA_LAUNCH_CHECK("attention_decode");
-    if (max_chunks > 1) {
-      dim3 mg(Hq, n);
-      flash_decode_merge_kernel<<<mg, RA_WAVE, 0, stream>>>(po, pm, (bf16_t*)out, out_stride, list, positions,
-                                                           Hkv, G, d, window, chunk_shift, max_chunks, base);
-      RA_LAUNCH_CHECK("attention_decode merge");
-    }
+  RA_LAUNCH_CHECK("attention_decode");
+  if (max_chunks > 1) {
+    RA_CHECK(n_tokens <= 65535, "attention_decode: %d tokens in one launch of the merge (max 65535)", n_tokens);
+    dim3 mg(Hq, n_tokens);
+#define RA_FDM(AH)                                                                                          \
+  flash_decode_merge_kernel<AH><<<mg, RA_WAVE, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, token_list, \
+                                                           positions, Hkv, G, d, window, chunk_shift, max_chunks, 0)
+    if (max_chunks > FDM_AHEAD) RA_FDM(0);
+    else if (d <= 64) RA_FDM(1);
+    else if (d <= 128) RA_FDM(2);
+    else RA_FDM(4);
+#undef RA_FDM
+    RA_LAUNCH_CHECK("attention_decode merge");
   }
   return 0;
 }

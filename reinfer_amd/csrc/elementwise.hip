@@ -298,6 +298,98 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
   }
 }
 
+// The same for few tokens of the common shape (half-split rotation over the whole head, head size 64,
+// 128 or 256, the product already added): one wave per (token, head), and one trip to memory. A decode
+// step's launch of this kernel does almost no work, so its time is the trips to memory that wait for
+// each other; here the token's slot and position, the head's elements, the norm weights and the
+// frequencies are all asked for before the first of them is used. A lane holds elements lane + 64 k: for
+// EPL >= 2 both members of its rotation pairs (j, j + d/2); for EPL = 1 the partner sits 32 lanes away.
+// An element as its bits in a register of its own: nothing is computed on a loaded value (a conversion,
+// a packing of two halves) before the last load is out.
+__device__ __forceinline__ unsigned raw_bits(const float* p, int i) { return ((const unsigned*)p)[i]; }
+__device__ __forceinline__ unsigned raw_bits(const bf16_t* p, int i) { return (unsigned)((const unsigned short*)p)[i]; }
+template <typename T> __device__ __forceinline__ float raw_value(unsigned bits);
+template <> __device__ __forceinline__ float raw_value<float>(unsigned bits) { return __uint_as_float(bits); }
+template <> __device__ __forceinline__ float raw_value<bf16_t>(unsigned bits) { return __uint_as_float(bits << 16); }
+
+template <typename TA, typename TW, int EPL, bool NORM>
+__global__ void __launch_bounds__(QK_WAVES * RA_WAVE)
+qk_norm_rope_cache_head_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w, const TW* __restrict__ k_w,
+                               float eps, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                               const int* __restrict__ slots, TA* __restrict__ kcache, TA* __restrict__ vcache,
+                               int block_size, int Hq, int Hkv) {
+  constexpr int d = 64 * EPL, half = d / 2;
+  constexpr int NF = EPL >= 2 ? EPL / 2 : 1;
+  const int lane = threadIdx.x & (RA_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / RA_WAVE);      // the same in every lane
+  const int t = blockIdx.y;
+  const int head = blockIdx.x * QK_WAVES + wave;
+  const int n_heads = Hq + 2 * Hkv;
+  if (head >= n_heads) return;
+  TA* u = qkv + ((size_t)t * n_heads + head) * d;
+  const bool is_q = head < Hq;
+  const bool is_k = !is_q && head < Hq + Hkv;
+  const TW* w = is_q ? q_w : k_w;              // a v head reads k's weights and drops them
+  // ---- every load, then the first use
+  const int slot = slots[t];
+  const int posi = positions[t];
+  unsigned xr[EPL], wr[EPL];
+  float fr[NF];
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) xr[k] = raw_bits(u, lane + 64 * k);
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) wr[k] = NORM ? raw_bits(w, lane + 64 * k) : 0u;
+#pragma unroll
+  for (int k = 0; k < NF; ++k) fr[k] = inv_freq[EPL >= 2 ? lane + 64 * k : (lane & 31)];
+  asm volatile("" ::: "memory");               // no load moves below this line, into the branches that follow
+  // ----
+  const int kvh = is_q ? 0 : (is_k ? head - Hq : head - Hq - Hkv);
+  if (!is_q && slot < 0) return;               // nothing to store for this token
+  const size_t blk = slot >= 0 ? (size_t)(slot / block_size) : 0;
+  const int off = slot >= 0 ? slot % block_size : 0;
+  TA* slab = is_q ? nullptr : (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d;
+  float x[EPL];
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) x[k] = raw_value<TA>(xr[k]);
+  if (!is_q && !is_k) {                        // v head: copy into the V tile order
+#pragma unroll
+    for (int k = 0; k < EPL; ++k) slab[cache_v_index(off, lane + 64 * k, d)] = from_f32<TA>(x[k]);
+    return;
+  }
+  if (NORM) {
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < EPL; ++k) ss += x[k] * x[k];
+    ss = wave_sum(ss);
+    const float rstd = rsqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < EPL; ++k) x[k] = x[k] * rstd * raw_value<TW>(wr[k]);
+  }
+  const float pos = (float)posi;
+  float y[EPL];
+  if (EPL >= 2) {
+#pragma unroll
+    for (int k = 0; k < NF; ++k) {             // pair (lane + 64 k, lane + 64 k + d/2)
+      float sn, cs;
+      sincosf(pos * fr[k], &sn, &cs);
+      const float a = x[k], c = x[k + NF];
+      y[k] = a * cs - c * sn;
+      y[k + NF] = a * sn + c * cs;
+    }
+  } else {
+    float sn, cs;
+    sincosf(pos * fr[0], &sn, &cs);
+    const float other = __shfl_xor(x[0], 32, RA_WAVE);
+    y[0] = lane < 32 ? x[0] * cs - other * sn : other * sn + x[0] * cs;
+  }
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) {
+    const int i = lane + 64 * k;
+    if (is_q) u[i] = from_f32<TA>(y[k]);
+    else slab[cache_k_index(off, i, d)] = from_f32<TA>(y[k]);
+  }
+}
+
 // The same for the common shape (half-split rotation over the whole head, head
 // size a power of two between 16 and 256): one workgroup per token. The sines and
 // cosines of the token's angles are computed once, in LDS, for all heads (the
@@ -407,6 +499,33 @@ static int qk_norm_rope_cache_impl(void* qkv, int act_dtype, const void* q_weigh
     return 0;
   }
   dim3 grid((Hq + 2 * Hkv + QK_WAVES - 1) / QK_WAVES, n_tokens);
+  if (!sm.parts && (d == 64 || d == 128 || d == 256) && rope_style == 0 && rotary_dim == d) {
+#define RA_HEAD2(TA, TW, EPL)                                                                             \
+  do {                                                                                                    \
+    if (q_weight)                                                                                         \
+      qk_norm_rope_cache_head_kernel<TA, TW, EPL, true><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(         \
+          (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, slots, (TA*)kcache, \
+          (TA*)vcache, block_size, Hq, Hkv);                                                              \
+    else                                                                                                  \
+      qk_norm_rope_cache_head_kernel<TA, TW, EPL, false><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(        \
+          (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, slots, (TA*)kcache, \
+          (TA*)vcache, block_size, Hq, Hkv);                                                              \
+  } while (0)
+#define RA_HEAD(TA, TW)                      \
+  do {                                       \
+    if (d == 64) RA_HEAD2(TA, TW, 1);        \
+    else if (d == 128) RA_HEAD2(TA, TW, 2);  \
+    else RA_HEAD2(TA, TW, 4);                \
+  } while (0)
+    if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_HEAD(float, float);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_HEAD(bf16_t, bf16_t);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_HEAD(bf16_t, float);
+    else return ra_fail("qk_norm_rope_cache: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
+#undef RA_HEAD
+#undef RA_HEAD2
+    RA_LAUNCH_CHECK("qk_norm_rope_cache");
+    return 0;
+  }
 #define RA_GO(TA, TW)                                                                              \
   qk_norm_rope_cache_kernel<TA, TW><<<grid, QK_WAVES * RA_WAVE, 0, stream>>>(                      \
       (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, rotary_dim,   \
