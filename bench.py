@@ -11,7 +11,8 @@ run through the engine's own loop (scheduler, step function, GPU sampler). One
 JSON line goes to standard output: ``value`` is decoded tokens a second at batch
 8; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the
 decode step against 8 TB/s by the bytes it must read (every weight once and the
-keys and values of the live requests); ``points`` holds batch 1 and batch 64.
+keys and values of the live requests); ``points`` holds batch 1 and batch 64;
+``kernel_ms`` the decode step's GPU time by kernel class with the bytes each class reads.
 ``--serve N`` runs a continuous-batching workload of N requests instead (the reference's replay harness
 feeds its scheduler synthetic arrivals the same way, crates/scheduler/src/replay.rs:180-217).
 ``--shape 4b`` and ``--shape 32b`` run the same measurement at the Qwen3-4B and Qwen3-32B layer sizes.
@@ -118,6 +119,62 @@ def prefill_run(engine, raw, tokens: int, reps: int, seed: int) -> float:
     return statistics.median(times)
 
 
+def profile_run(engine, raw, batch: int, prompt_len: int, steps: int, seed: int, max_tokens: int, elem: int):
+    """GPU time of a decode step by kernel class: ``steps`` steps run without the captured graph, every call
+    into the kernel set between two events, queued behind work that keeps the GPU busy meanwhile so that the
+    kernels run back to back as they do in a replayed graph. -> class -> {"ms", "calls", "bytes", "flops"} a
+    step (``bytes``: what the class must read, ``flops``: its products; 0 where neither says much)."""
+    import torch
+    from reinfer_amd import kernels
+    from reinfer_amd.kernels.profile import TimedKernels
+    from reinfer_amd.sampling import SamplingParams
+    g = torch.Generator().manual_seed(seed)
+    params = SamplingParams(temperature=0.0, max_tokens=max_tokens, ignore_eos=True)
+    rids = [engine.add_request(torch.randint(0, raw["vocab_size"], (prompt_len,), generator=g).tolist(), params)
+            for _ in range(batch)]
+    sched = engine.scheduler
+    while any(not r.decoding for r in sched.running) or sched.waiting:
+        engine.step()
+    engine.step()
+    model = engine.runner.model
+    timed = TimedKernels(kernels.current())
+    for b in model.blocks:
+        for part, attr, role in ((getattr(b, "mixer", None), "w_qkv", "qkv"), (getattr(b, "mixer", None), "w_o", "o_proj"),
+                                 (getattr(b, "ffn", None), "w_gate_up", "gate_up"), (getattr(b, "ffn", None), "w_down", "down")):
+            w = getattr(part, attr, None)
+            if w is not None:
+                timed.name_weight(w, role)
+    timed.name_weight(model.head, "head")
+    graphs, engine.runner.graphs = engine.runner.graphs, None
+    try:
+        with kernels.use(timed):
+            for _ in range(steps):
+                timed.hold_back(25.0, engine.device)
+                engine.step()
+        rows = timed.report()
+    finally:
+        engine.runner.graphs = graphs
+    ctx = statistics.mean(r.num_tokens for r in sched.running)
+    for r in rids:
+        engine.abort(r)
+    h, L, I, V = raw["hidden_size"], raw["num_hidden_layers"], raw["intermediate_size"], raw["vocab_size"]
+    nq = raw["num_attention_heads"] * raw["head_dim"]
+    nkv = raw["num_key_value_heads"] * raw["head_dim"]
+    weights = {"qkv": L * h * (nq + 2 * nkv), "o_proj": L * nq * h, "gate_up": L * 2 * h * I, "down": L * I * h,
+               "head": V * h}
+    out = {}
+    for label, row in sorted(rows.items(), key=lambda kv: -kv[1]["ms"]):
+        rec = {"ms": round(row["ms"] / steps, 4), "calls": round(row["calls"] / steps, 1), "bytes": 0, "flops": 0}
+        if label in weights:
+            rec["bytes"] = weights[label] * elem
+            rec["flops"] = 2 * batch * weights[label]
+        elif label == "attention":
+            rec["bytes"] = int(batch * ctx * kv_bytes_per_token(raw, elem))
+            rec["flops"] = int(4 * batch * ctx * nq * L)
+        out[label] = rec
+    return out
+
+
 def serve_run(args, raw, shape_name: str) -> int:
     """Continuous batching: ``args.serve`` requests arrive at once, prompts uniform in [64, 4096] tokens and
     outputs uniform in [32, 512], prompts cut into portions under a 2,048-token step budget beside the
@@ -179,6 +236,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-profile", action="store_true", help="skip the per-kernel-class times of the decode step")
+    ap.add_argument("--profile-steps", type=int, default=4, help="decode steps timed kernel by kernel")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--serve", type=int, default=0, metavar="REQUESTS",
                     help="instead of the decode measurement: continuous batching of this many requests")
@@ -265,6 +324,14 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
             log(f"decode batch {b}: {pms:.3f} ms a step, {points[f'decode_b{b}']:.0f} tok/s")
 
+    kernel_ms = None
+    if not args.no_profile:
+        kernel_ms = profile_run(engine, raw, args.batch, args.prompt_len, args.profile_steps, args.seed + 90, max_new, elem)
+        total = sum(r["ms"] for r in kernel_ms.values())
+        log(f"decode batch {args.batch}, kernel by kernel (events, no graph): {total:.3f} ms a step: " +
+            ", ".join(f"{k} {r['ms'] * 1e3:.0f} us" + (f" ({r['bytes'] / r['ms'] / 1e6:.0f} GB/s)" if r["bytes"] else "")
+                      for k, r in kernel_ms.items()))
+
     peaks = kernels.current().measure_peaks(engine.device)
     log(f"measured on this GPU: a plain read {peaks['hbm_read_GBps']:.0f} GB/s, bfloat16 matrix cores "
         f"{peaks['mfma_bf16_32x32x16_TFLOPs']:.0f} TFLOP/s with 32x32x16 products, {peaks['mfma_bf16_16x16x32_TFLOPs']:.0f} with "
@@ -287,6 +354,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        # GPU time of the decode step by kernel class (events around every kernel, outside the captured graph)
+        "kernel_ms": kernel_ms,
         # what this GPU gives at best, beside the published peaks that the fractions above use
         "measured_peaks": {k: round(v, 1) for k, v in peaks.items()},
     }

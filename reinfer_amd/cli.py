@@ -48,6 +48,8 @@ def _add_run_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("--perf", action="store_true", help="print a machine-parseable perf line")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--block-size", type=int, default=16)
+    p.add_argument("--allow-extra-tensors", action="store_true",
+                   help="leave tensors of the folder that the model does not declare unread instead of refusing them")
     p.add_argument("--num-blocks", type=int, default=None, help="cache blocks (default: from free memory)")
     p.add_argument("--max-num-seqs", type=int, default=64)
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
@@ -93,7 +95,11 @@ def cmd_run(args) -> int:
     engine = LLMEngine(args.model, dtype=args.dtype, max_model_len=args.max_model_len,
                        block_size=args.block_size, num_blocks=args.num_blocks,
                        max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
-                       seed=args.seed or 0)
+                       seed=args.seed or 0, allow_unexpected=args.allow_extra_tensors)
+    extra = engine.runner.load_report.get("unexpected") or []
+    if extra:
+        print(f"reinfer: {len(extra)} tensors of the folder are not part of the model and were left unread "
+              f"({', '.join(extra[:4])}{', ...' if len(extra) > 4 else ''})", file=sys.stderr)
     t_load = time.perf_counter() - t_load
     tokenizer = _load_tokenizer(args.model)
     ids = _prompt_ids(args, engine.runner.spec.vocab_size, tokenizer)

@@ -111,6 +111,7 @@ class _CapturedStep:
             "prefill_list": None, "n_tiles": 0, "tiles": None}
         self.logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.copied: Optional[torch.cuda.Event] = None      # behind the last copy out of the staging buffer
         self._capture(pool)
 
     def _body(self) -> None:
@@ -144,10 +145,18 @@ class _CapturedStep:
                 gc.enable()
 
     def fill(self, entries: List[StepEntry], sampling) -> None:
+        # The staging buffer is the source of the last replay's copy, which the GPU may not have made
+        # yet if nobody read that step's results (a step with no logits wanted): wait for that copy
+        # before the buffer is written again, or the last step would run with this step's indices.
+        if self.copied is not None:
+            self.copied.synchronize()
         self.rows.fill(entries, self.h, sampling)
 
     def replay(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
         self.graph.replay()
 
 

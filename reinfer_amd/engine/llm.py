@@ -42,12 +42,13 @@ class LLMEngine:
                  max_model_len: Optional[int] = None, block_size: int = 16,
                  num_blocks: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, max_chunk: Optional[int] = None,
-                 memory_fraction: float = 0.9, admission: str = "peak"):
+                 memory_fraction: float = 0.9, admission: str = "peak", allow_unexpected: bool = False):
         limits = dict(block_size=block_size, num_blocks=num_blocks, max_seqs=max_num_seqs,
                       max_model_len=max_model_len, memory_fraction=memory_fraction)
         if model is not None:
             self.config = load_config(model)
-            self.runner = ModelRunner.from_folder(model, dtype=dtype, device=device, **limits)
+            self.runner = ModelRunner.from_folder(model, dtype=dtype, device=device,
+                                                  allow_unexpected=allow_unexpected, **limits)
         elif config is not None:
             self.config = config
             self.runner = ModelRunner.from_config(config, seed=seed, dtype=dtype, device=device,
@@ -139,6 +140,10 @@ class LLMEngine:
                 first = time.perf_counter() - t0
         self.timings = {"total_s": time.perf_counter() - t0, "first_step_s": first or 0.0}
         return [outs[r] for r in rids]
+
+    def get_weight(self, name: str) -> torch.Tensor:
+        """The tensor ``name`` as the model was given it, on the CPU (see ModelRunner.get_weight)."""
+        return self.runner.get_weight(name)
 
     def cache_stats(self) -> Dict[str, object]:
         s = self.runner.manager.stats()

@@ -18,7 +18,7 @@ from ..config import load_config
 from ..config.schema import ModelSpec
 from ..models import DecoderModel, declare_params
 from ..parts import KVNeed, LayerCache, StateNeed
-from ..weights import check_tensors, load_weights, random_tensors, storage_dtype
+from ..weights import check_tensors, load_weights, random_tensor, random_tensors, storage_dtype, weight_from_folder
 from .._hostlib import StepError
 from .batch import StepBatch, StepEntry, build_step_batch
 from .graphs import MAX_GRAPH_BATCH
@@ -47,6 +47,8 @@ class ModelRunner:
         self.spec = spec
         self.dtype = dtype
         self.device = device
+        self._weight_source = ("given", weights)       # replaced by from_folder / from_config; see get_weight
+        self.load_report: Dict[str, object] = {}
         self.block_size = int(block_size)
         self.max_model_len = min(max_model_len or spec.max_positions, spec.max_positions)
         self.max_seqs = int(max_seqs)
@@ -110,13 +112,20 @@ class ModelRunner:
 
     # ------------------------------------------------------------ building
     @classmethod
-    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **limits) -> "ModelRunner":
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", allow_unexpected: bool = False,
+                    **limits) -> "ModelRunner":
+        """``allow_unexpected``: tensors of the folder that the model does not declare are left unread
+        (``load_report["unexpected"]`` names them) instead of refused."""
         cfg = load_config(model_dir)
         spec = cfg.to_spec()
         tdtype = parse_dtype(dtype)
         dev = torch.device(device)
-        weights = load_weights(model_dir, declare_params(spec), tdtype, dev)
-        return cls(spec, weights, tdtype, dev, **limits)
+        report: Dict[str, object] = {}
+        weights = load_weights(model_dir, declare_params(spec), tdtype, dev, allow_unexpected, report)
+        runner = cls(spec, weights, tdtype, dev, **limits)
+        runner._weight_source = ("folder", model_dir)
+        runner.load_report = report
+        return runner
 
     @classmethod
     def from_config(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0",
@@ -126,13 +135,37 @@ class ModelRunner:
         tdtype = parse_dtype(dtype)
         dev = torch.device(device)
         decls = declare_params(spec)
+        source = ("seed", int(seed))
         if weights is None:
             weights = random_tensors(decls, seed, tdtype, dev)
         else:
             check_tensors("weights", decls, weights)
             by = {d.name: d for d in decls}
+            source = ("given", weights)
             weights = {n: t.to(storage_dtype(by[n], t.dtype, tdtype)).to(dev) for n, t in weights.items()}
-        return cls(spec, weights, tdtype, dev, **limits)
+        runner = cls(spec, weights, tdtype, dev, **limits)
+        runner._weight_source = source
+        return runner
+
+    def get_weight(self, name: str) -> torch.Tensor:
+        """The tensor ``name`` as the model was given it (before any fusing or re-laying by the parts), on
+        the CPU: read from the folder again, drawn again from the seed, or the caller's own tensor. For
+        checking the engine against another implementation with the very same weights
+        (crates/cuda/tests/engine_vs_cpu.rs:80-118 reads them back for that)."""
+        decls = {d.name: d for d in declare_params(self.spec)}
+        if name not in decls:
+            raise KeyError(f"{name}: the model declares no such tensor")
+        kind, what = self._weight_source
+        if kind == "folder":
+            return weight_from_folder(what, name)
+        if kind == "seed":
+            d = decls[name]
+            if d.optional:
+                raise KeyError(f"{name}: not part of this random model (a tied head)")
+            return random_tensor(d, what, self.dtype)
+        if name not in what:
+            raise KeyError(f"{name}: not among the tensors the model was built from")
+        return what[name].detach().cpu()
 
     def _blocks_that_fit(self, needs, windows, fraction: float) -> int:
         """Blocks per group from free device memory: the reference's budget,
@@ -168,13 +201,15 @@ class ModelRunner:
         return self.manager.get(rid).num_tokens
 
     # --------------------------------------------------------------- step
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], observer=None) -> torch.Tensor:
         """Run the entries' tokens as one batch; logits [wanted, vocab] float32,
         in the order of the entries and of each entry's ``want``. The result may be
-        a view of a buffer that the next step overwrites: use it before stepping again."""
-        return self.step_sampled(entries, None)[0]
+        a view of a buffer that the next step overwrites: use it before stepping again.
+        ``observer(i, hidden)`` sees the hidden state of all the step's tokens behind the embedding
+        and behind every layer (such a step never replays a captured graph)."""
+        return self.step_sampled(entries, None, observer)[0]
 
-    def step_sampled(self, entries: Sequence[StepEntry], sampling=None):
+    def step_sampled(self, entries: Sequence[StepEntry], sampling=None, observer=None):
         """As :meth:`step`; ``sampling`` = (temperatures, seeds, positions), one per entry,
         asks for a token from each entry's single wanted row where the step can draw it
         itself. -> (logits, tokens): ``tokens`` is an int32 device tensor, one per
@@ -185,7 +220,7 @@ class ModelRunner:
         one_token, one_want, longest = self.manager.begin_step(entries, self.spec.vocab_size,
                                                                self.max_model_len)
         tokens = None
-        if self.graphs is not None and one_token and len(entries) <= MAX_GRAPH_BATCH:
+        if self.graphs is not None and one_token and len(entries) <= MAX_GRAPH_BATCH and observer is None:
             all_logits, all_tokens = self.graphs.run(entries, longest, sampling)
             n = len(entries)
             if one_want:
@@ -198,17 +233,14 @@ class ModelRunner:
                     else all_logits[:0]
         else:
             batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
-            logits = self.forward(batch)
+            logits = self.forward(batch, observer)
         self.manager.end_step(entries)
         return logits, tokens
 
-    def forward(self, batch: StepBatch) -> torch.Tensor:
+    def forward(self, batch: StepBatch, observer=None) -> torch.Tensor:
         with torch.no_grad():
             if batch.num_logit_rows == 0:
                 # still run the layers: the step's keys and values must be stored
-                self._forward_no_logits(batch)
+                self.model.forward_layers(batch, self.caches, observer)
                 return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-            return self.model.forward(batch, self.caches)
-
-    def _forward_no_logits(self, batch: StepBatch) -> None:
-        self.model.forward_layers(batch, self.caches)
+            return self.model.forward(batch, self.caches, observer)

@@ -53,11 +53,17 @@ class DecoderModel:
             needs.append(need)
         return needs
 
-    def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]]):
-        """Embedding and all blocks: (residual stream, last addend not yet added)."""
+    def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]], observer=None):
+        """Embedding and all blocks: (residual stream, last addend not yet added).
+
+        ``observer(i, hidden)``, if given, is called with the float32 hidden state [T, hidden] behind
+        the embedding (i = 0) and behind run-order entry i - 1 (the reference reads activations back
+        layer by layer the same way, crates/cuda/src/engine.rs:3744-3765)."""
         ops = kernels.current()
         resid = torch.empty((batch.num_tokens, self.spec.hidden), dtype=torch.float32, device=self.device)
         ops.embed(self.embed, batch.token_ids, resid)
+        if observer is not None:
+            observer(0, resid.clone())
         delta = None
         n = len(self.run_order)
         for i, e in enumerate(self.run_order):
@@ -73,14 +79,17 @@ class DecoderModel:
                 delta = block.forward(resid, delta, batch, caches[i], emit=tgt)
             else:
                 delta = block.forward(resid, delta, batch, caches[i])
+            if observer is not None:
+                # the block's last addend may not be in the stream yet
+                observer(i + 1, resid + delta.float() if isinstance(delta, torch.Tensor) else resid.clone())
         return resid, delta
 
-    def forward(self, batch, caches: Sequence[Optional[LayerCache]]) -> torch.Tensor:
+    def forward(self, batch, caches: Sequence[Optional[LayerCache]], observer=None) -> torch.Tensor:
         """Logits [len(batch.logit_rows), vocab] in float32 for the step's tokens.
 
         The head runs on the wanted rows only (the reference computes all rows of
         a prompt and keeps the last, crates/cuda/src/engine.rs:5685-5720)."""
-        resid, delta = self.forward_layers(batch, caches)
+        resid, delta = self.forward_layers(batch, caches, observer)
         if delta is not None and not isinstance(delta, torch.Tensor):
             delta = None               # a filled norm target: the sum is already in the stream
         xn = self.final_norm.add_norm(resid, delta, rows=batch.logit_rows)

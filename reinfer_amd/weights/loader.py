@@ -95,12 +95,21 @@ def _open_folder(model_dir: str) -> Tuple[Dict[str, SafetensorsFile], Dict[str, 
 
 
 def load_weights(model_dir: str, decls: Sequence[ParamDecl], compute_dtype: torch.dtype,
-                 device: torch.device) -> Dict[str, torch.Tensor]:
+                 device: torch.device, allow_unexpected: bool = False,
+                 report: Optional[Dict[str, object]] = None) -> Dict[str, torch.Tensor]:
+    """Tensors that no part declares are an error like the others (a folder that holds another model's
+    tensors is more often a mistake than an exporter's extras); with ``allow_unexpected`` they are
+    left unread, as the reference leaves what it does not ask for (crates/cuda/src/engine.rs:3216-3235),
+    and ``report["unexpected"]`` lists them."""
     files, where = _open_folder(model_dir)
     try:
         wanted = {d.name: d for d in decls}
         missing = [d.name for d in decls if d.name not in where and not d.optional]
         unexpected = [n for n in where if n not in wanted and not n.endswith(_IGNORABLE_SUFFIXES)]
+        if report is not None:
+            report["unexpected"] = list(unexpected)
+        if allow_unexpected:
+            unexpected = []
         wrong_shape, wrong_dtype = [], []
         for d in decls:
             if d.name not in where:
@@ -125,6 +134,18 @@ def load_weights(model_dir: str, decls: Sequence[ParamDecl], compute_dtype: torc
             t = files[where[d.name]].tensor(d.name)
             out[d.name] = t.to(storage_dtype(d, t.dtype, compute_dtype)).to(device)
         return out
+    finally:
+        for f in files.values():
+            f.close()
+
+
+def weight_from_folder(model_dir: str, name: str) -> torch.Tensor:
+    """One tensor of a model folder, as stored, on the CPU."""
+    files, where = _open_folder(model_dir)
+    try:
+        if name not in where:
+            raise KeyError(f"{model_dir}: no tensor {name}")
+        return files[where[name]].tensor(name).clone()
     finally:
         for f in files.values():
             f.close()

@@ -1,8 +1,9 @@
 """Random-weights mode: a model folder from a configuration and a seed.
 
-Every tensor has a generator of its own, seeded from (seed, tensor name), so a
-tensor's values do not depend on which other tensors exist. Matrices and the
-embedding are N(0, 0.02); norm weights U(0.8, 1.2). The reference has no such
+Every element is a function of (seed, tensor name, index): a tensor's values do
+not depend on which other tensors exist or on the device that draws them.
+Matrices and the embedding are bell-shaped with deviation 0.02; norm weights
+uniform on [0.8, 1.2). The reference has no such
 mode (its tests need a real checkpoint, scripts/ci/ignored-tests.txt).
 """
 from __future__ import annotations
@@ -38,31 +39,71 @@ def tensor_seed(seed: int, name: str) -> int:
     return splitmix64((seed & _MASK) ^ _fnv1a(name)) & ((1 << 63) - 1)
 
 
+_CHUNK = 1 << 24        # elements drawn at a time: bounds the temporaries of a large matrix
+
+
+def _mix(z: torch.Tensor) -> torch.Tensor:
+    """The finalising stage of SplitMix64 on int64 tensors (products wrap, shifts made logical by a mask)."""
+    z = (z ^ ((z >> 30) & 0x3FFFFFFFF)) * -0x40A7B892E31B1A47         # 0xBF58476D1CE4E5B9 as a signed value
+    z = (z ^ ((z >> 27) & 0x1FFFFFFFFF)) * -0x6B2FB644ECCEEE15         # 0x94D049BB133111EB
+    return z ^ ((z >> 31) & 0x1FFFFFFFF)
+
+
+def _signed(x: int) -> int:
+    x &= _MASK
+    return x - (1 << 64) if x >= (1 << 63) else x
+
+
+def _draw(n: int, seed: int, kind: str, device: torch.device, std: float) -> torch.Tensor:
+    """Element i of a tensor is a function of (seed, i) alone, made of integer operations and one float
+    product, so the CPU and the GPU draw the same bits. "normal": the sum of eight 16-bit fields of two
+    hashed words, centred and scaled to the standard deviation (a bell over +-4.9 deviations);
+    "uniform": 24 bits over [0.8, 1.2)."""
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    for lo in range(0, n, _CHUNK):
+        hi = min(n, lo + _CHUNK)
+        i = torch.arange(lo, hi, dtype=torch.int64, device=device)
+        a = _mix(i * 2 + _signed(seed) + _signed(0x9E3779B97F4A7C15))
+        if kind == "normal":
+            b = _mix(i * 2 + 1 + _signed(seed) + _signed(0x9E3779B97F4A7C15))
+            s = torch.zeros_like(i)
+            for word in (a, b):
+                for shift in (0, 16, 32, 48):
+                    s += (word >> shift) & 0xFFFF
+            # eight uniform fields on 0..65535: mean 4 * 65535, variance 8 * (65536^2 - 1) / 12
+            scale = std / (((65536.0 ** 2 - 1.0) * 8.0 / 12.0) ** 0.5)
+            out[lo:hi] = (s - 4 * 65535).to(torch.float32) * scale
+        else:
+            out[lo:hi] = 0.8 + ((a >> 40) & 0xFFFFFF).to(torch.float32) * (0.4 / 16777216.0)
+    return out
+
+
+def random_tensor(decl: ParamDecl, seed: int, dtype: torch.dtype,
+                  device: torch.device = torch.device("cpu"), std: float = 0.02) -> torch.Tensor:
+    """One declared tensor of the random model of ``seed``: drawn in float32, rounded once to ``dtype``;
+    the same values on every device."""
+    n = 1
+    for v in decl.shape:
+        n *= int(v)
+    if decl.init == "normal":
+        t = _draw(n, tensor_seed(seed, decl.name), "normal", device, std).view(decl.shape)
+    elif decl.init == "norm":
+        t = _draw(n, tensor_seed(seed, decl.name), "uniform", device, std).view(decl.shape)
+    elif decl.init == "zeros":
+        t = torch.zeros(decl.shape, dtype=torch.float32, device=device)
+    elif decl.init == "int":
+        t = torch.zeros(decl.shape, dtype=torch.int32, device=device)
+    else:
+        raise ValueError(f"{decl.name}: unknown init {decl.init!r}")
+    return t if decl.role == INT_TABLE else t.to(dtype)
+
+
 def random_tensors(decls: Sequence[ParamDecl], seed: int, dtype: torch.dtype,
                    device: torch.device = torch.device("cpu"), std: float = 0.02) -> Dict[str, torch.Tensor]:
-    """Values are drawn in float32 and rounded once to ``dtype``.
-
-    The stream of a generator differs between device kinds, so a folder (always
-    drawn on the CPU) is what makes a model reproducible, not the seed alone.
-    """
-    out: Dict[str, torch.Tensor] = {}
-    for d in decls:
-        if d.optional:
-            continue
-        g = torch.Generator(device=device)
-        g.manual_seed(tensor_seed(seed, d.name))
-        if d.init == "normal":
-            t = torch.empty(d.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=g)
-        elif d.init == "norm":
-            t = torch.empty(d.shape, dtype=torch.float32, device=device).uniform_(0.8, 1.2, generator=g)
-        elif d.init == "zeros":
-            t = torch.zeros(d.shape, dtype=torch.float32, device=device)
-        elif d.init == "int":
-            t = torch.zeros(d.shape, dtype=torch.int32, device=device)
-        else:
-            raise ValueError(f"{d.name}: unknown init {d.init!r}")
-        out[d.name] = t if d.role == INT_TABLE else t.to(dtype)
-    return out
+    """Every declared tensor (but the optional ones) of the random model of ``seed``. A value depends on
+    the seed, the tensor's name and the element's index, not on the device or on what else is drawn: a
+    model drawn on the GPU is the one a folder written on the CPU holds."""
+    return {d.name: random_tensor(d, seed, dtype, device, std) for d in decls if not d.optional}
 
 
 def write_model_folder(config, seed: int, out_dir: str, dtype: str = "bfloat16") -> str:

@@ -127,14 +127,32 @@ def layer_windows(cfg: Mapping) -> List[int]:
 
 
 def forward(cfg: Mapping, weights: Mapping[str, torch.Tensor], tokens: Sequence[int],
-            dtype: torch.dtype = torch.float64, start_pos: int = 0) -> torch.Tensor:
-    """Logits [T, V] of one whole sequence.
+            dtype: torch.dtype = torch.float64, start_pos: int = 0,
+            rows: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Logits [T, V] of one whole sequence (with ``rows``: of those positions only, [len(rows), V]; the
+    layers still run every position, only the head's product is smaller).
 
     Order of work: crates/cuda/tests/engine_vs_cpu.rs:162-281 (embedding row,
     per layer: norm, attention, residual add, norm, SwiGLU, residual add; final
     norm; head). Tied head: the embedding matrix (crates/cpu/src/model.rs:218-225).
     ``start_pos`` shifts all positions (only distances count in the result).
     """
+    x = hidden_states(cfg, weights, tokens, dtype, start_pos)[-1]
+    w = {k: weights[k].to(dtype) for k in ("model.norm.weight", "model.embed_tokens.weight", "lm_head.weight")
+         if k in weights}
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    if rows is not None:
+        x = x[torch.tensor(list(rows), dtype=torch.long)]
+    xn = rms_norm(x, w["model.norm.weight"], eps)
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
+    return xn @ head.T
+
+
+def hidden_states(cfg: Mapping, weights: Mapping[str, torch.Tensor], tokens: Sequence[int],
+                  dtype: torch.dtype = torch.float64, start_pos: int = 0) -> List[torch.Tensor]:
+    """The hidden state [T, hidden] behind the embedding and behind every layer (layers + 1 tensors):
+    what the reference reads back layer by layer when it looks for the first layer that differs
+    (crates/cuda/src/engine.rs:3744-3765); same order of work as :func:`forward`."""
     w = {k: v.to(dtype) for k, v in weights.items()}
     h = cfg["hidden_size"]
     Hq = cfg["num_attention_heads"]
@@ -146,6 +164,7 @@ def forward(cfg: Mapping, weights: Mapping[str, torch.Tensor], tokens: Sequence[
     ids = torch.tensor(list(tokens), dtype=torch.long)
     positions = torch.arange(len(tokens)) + start_pos
     x = w["model.embed_tokens.weight"][ids]
+    out = [x]
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
         xn = rms_norm(x, w[p + "input_layernorm.weight"], eps)
@@ -153,9 +172,8 @@ def forward(cfg: Mapping, weights: Mapping[str, torch.Tensor], tokens: Sequence[
         xn = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
         x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                        w[p + "mlp.down_proj.weight"])
-    xn = rms_norm(x, w["model.norm.weight"], eps)
-    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
-    return xn @ head.T
+        out.append(x)
+    return out
 
 
 def argmax_first(logits: torch.Tensor) -> int:

@@ -234,3 +234,60 @@ def test_no_size_stands_in_code():
     assert decls["model.layers.0.self_attn.k_norm.weight"] == (24,)
     assert decls["model.layers.0.mlp.down_proj.weight"] == (40, 56)
     assert decls["lm_head.weight"] == (123, 40)
+
+
+def test_unexpected_tensors_are_refused_unless_allowed(tmp_path):
+    """A tensor that no part declares is listed in the one error; with ``allow_unexpected`` it is left
+    unread and named in the report (the reference reads what it asks for and no more,
+    crates/cuda/src/engine.rs:3216-3235)."""
+    import torch
+    from reinfer_amd.models import declare_params
+    from reinfer_amd.weights import WeightError, load_weights, random_tensors, write_safetensors
+    cfg = config_from_dict(TINY_A)
+    decls = declare_params(cfg.to_spec())
+    tensors = random_tensors(decls, 0, torch.bfloat16)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)      # a known exporter's extra: always let through
+    tensors["model.extra_head.weight"] = torch.zeros(3, 3)
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as e:
+        load_weights(str(tmp_path / "m"), decls, torch.bfloat16, torch.device("cpu"))
+    assert e.value.unexpected == ["model.extra_head.weight"] and not e.value.missing
+    report = {}
+    got = load_weights(str(tmp_path / "m"), decls, torch.bfloat16, torch.device("cpu"), allow_unexpected=True,
+                       report=report)
+    assert report["unexpected"] == ["model.extra_head.weight"]
+    assert "model.extra_head.weight" not in got and len(got) == len([d for d in decls if not d.optional])
+    # what is missing or misshapen is still refused
+    del tensors["model.norm.weight"]
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as e:
+        load_weights(str(tmp_path / "m"), decls, torch.bfloat16, torch.device("cpu"), allow_unexpected=True)
+    assert e.value.missing == ["model.norm.weight"] and not e.value.unexpected
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """A tensor's values do not depend on what else is drawn, on how the drawing is cut into pieces, or
+    (checked on the GPU box) on the device; they have the asked deviation and range."""
+    import torch
+    import reinfer_amd.weights.random_init as ri
+    from reinfer_amd.weights import ParamDecl, random_tensor, random_tensors
+    a = ParamDecl("a.weight", (300, 257))
+    n = ParamDecl("n.weight", (1000,), init="norm", role="vector")
+    one = random_tensor(a, 5, torch.float32)
+    both = random_tensors([n, a], 5, torch.float32)
+    assert torch.equal(one, both["a.weight"])
+    assert not torch.equal(one, random_tensor(a, 6, torch.float32))
+    assert not torch.equal(one, random_tensor(ParamDecl("b.weight", (300, 257)), 5, torch.float32))
+    chunk = ri._CHUNK
+    try:
+        ri._CHUNK = 1000
+        assert torch.equal(one, random_tensor(a, 5, torch.float32))
+    finally:
+        ri._CHUNK = chunk
+    assert abs(one.std().item() - 0.02) < 5e-4 and abs(one.mean().item()) < 3e-4
+    assert one.abs().max().item() < 0.02 * 4.9
+    u = both["n.weight"]
+    assert 0.8 <= u.min().item() and u.max().item() < 1.2 and abs(u.mean().item() - 1.0) < 0.02
+    # rounded once: the bfloat16 tensor is the rounding of the float32 one
+    assert torch.equal(random_tensor(a, 5, torch.bfloat16), one.to(torch.bfloat16))

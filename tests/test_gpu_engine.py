@@ -142,6 +142,29 @@ def test_batch_order_does_not_matter(folders):
         assert rel_err(b[r], alone[r]) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_whose_logits_nobody_reads(folders, plain_cache, dtype):
+    """Single-token steps with nothing wanted, between steps that are read: nobody waits for such a
+    step's results, so the next step is packed while it may not have started; each must still run with
+    its own indices (the steps replay a captured graph from a staging buffer that is written again)."""
+    toks = random_tokens(90, vocab("B"), 77)
+    want = reference(folders, plain_cache, "B", dtype, toks)
+    runner = runner_for(folders, "B", dtype, max_tokens=512, max_seqs=4)
+    for rep in range(2):                       # the second request replays the graph the first captured
+        runner.add_request("x")
+        runner.step([StepEntry("x", toks[:40], [])])
+        got = {}
+        for p in range(40, 90):
+            out = runner.step([StepEntry("x", [toks[p]], [0] if p % 7 == 0 or p == 89 else [])])
+            if out.shape[0]:
+                got[p] = out[0].float().cpu()
+        runner.free_request("x")
+        assert len(got) == 8
+        for p, row in got.items():
+            assert rel_err(row[None], want[p][None]) < TOL[dtype], (rep, p)
+
+
+
 @pytest.mark.parametrize("which,n_req", [("A", 5), ("B", 70)])
 def test_decode_graphs_replay_like_eager_steps(folders, which, n_req):
     """Decode steps replay captured HIP graphs (one per batch-size and context bucket, library

@@ -1,13 +1,21 @@
-"""The serving kernels at the sizes they are built for: a model with the widths of the
-Qwen3-8B shape (4096 wide, 32 query heads over 8 KV heads of 128, feed-forward 12288,
-vocabulary 151936) but two layers, random weights. The 32-bit path of the same engine
-is the reference here (the tiny models pin that path to the plain implementation);
-the bfloat16 path must agree with it under every way of cutting the work, and with
-itself across cuts far more closely than bfloat16 rounding alone would demand."""
+"""The serving kernels at the sizes they are built for, against the plain implementation.
+
+Models with the widths of the Qwen3-8B shape (4096 wide, 32 query heads over 8 KV heads of 128,
+feed-forward 12288, vocabulary 151936; two layers), of the Qwen3-4B shape (2560 wide with a 4096-wide
+q projection, tied head; one layer) and of the Qwen3-32B shape (5120 wide, 64 query heads in groups
+of 8, feed-forward 25600; one layer), random weights. The reference is ``plain_qwen3.forward`` in
+float32 on the CPU with the very same tensors (drawn once, on the GPU, and copied; the generator
+gives the same values on either device), at the wanted positions only. Both precisions of the
+engine are compared with it under the ways of cutting the work that the product runs at these widths:
+whole prompts, the last tokens one by one, portions of changing size, requests mixed in one step, a
+2,048-token prompt in one step and in portions behind earlier context, and 17, 33 and 64 requests
+decoding together (the products over K ranges, the captured steps), metric and bounds as for the
+tiny models (crates/cuda/tests/parity.rs:22-27)."""
 import pytest
 import torch
 
-from helpers import random_tokens, rel_err
+import plain_qwen3 as plain
+from helpers import TOL, random_tokens, rel_err
 from reinfer_amd import kernels
 from reinfer_amd.config import config_from_dict
 from reinfer_amd.engine import ModelRunner, StepEntry
@@ -16,61 +24,226 @@ from reinfer_amd.weights import random_tensors
 
 pytestmark = pytest.mark.gpu
 
-RAW = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
-       "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
-       "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
-       "max_position_embeddings": 4096}
+
+def raw_config(layers, hidden, heads, inter, tied):
+    return {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": layers, "hidden_size": hidden,
+            "num_attention_heads": heads, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": inter,
+            "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": tied,
+            "max_position_embeddings": 4096}
+
+
+SHAPES = {"8b": raw_config(2, 4096, 32, 12288, False), "4b": raw_config(1, 2560, 32, 9728, True),
+          "32b": raw_config(1, 5120, 64, 25600, False)}
+
+
+class Width:
+    """One shape: the weights, a runner per precision, and the plain logits of sequences by name."""
+
+    def __init__(self, name: str, max_tokens: int, max_seqs: int):
+        assert kernels.current().name == "hip-gfx950"
+        self.raw = SHAPES[name]
+        cfg = config_from_dict(self.raw)
+        dev = torch.device("cuda:0")
+        weights = random_tensors(declare_params(cfg.to_spec()), 7, torch.bfloat16, dev)
+        self.cpu = {k: v.float().cpu() for k, v in weights.items()}
+        self.runners = {dt: ModelRunner.from_config(cfg, dtype=dt, device="cuda:0", weights=weights,
+                                                    max_tokens=max_tokens, max_seqs=max_seqs)
+                        for dt in ("float32", "bfloat16")}
+        self.seqs = {}
+        self._plain = {}
+
+    def seq(self, key: str, n: int, seed: int):
+        self.seqs.setdefault(key, random_tokens(n, self.raw["vocab_size"], seed))
+        return self.seqs[key]
+
+    def plain_rows(self, key: str, rows):
+        """Plain float32 logits of sequence ``key`` at ``rows``; a sequence's rows are computed once."""
+        rows = tuple(rows)
+        if (key, rows) not in self._plain:
+            self._plain[(key, rows)] = plain.forward(self.raw, self.cpu, self.seqs[key], torch.float32, rows=rows)
+        return self._plain[(key, rows)]
 
 
 @pytest.fixture(scope="module")
-def engines():
-    assert kernels.current().name == "hip-gfx950"
-    cfg = config_from_dict(RAW)
-    dev = torch.device("cuda:0")
-    weights = random_tensors(declare_params(cfg.to_spec()), 0, torch.bfloat16, dev)
-    out = {}
-    for dtype in ("float32", "bfloat16"):
-        out[dtype] = ModelRunner.from_config(cfg, dtype=dtype, device="cuda:0", weights=weights, max_tokens=1024,
-                                             max_seqs=8)
-    return out
+def w8():
+    w = Width("8b", max_tokens=64 * 384, max_seqs=64)
+    yield w
+    del w
+    torch.cuda.empty_cache()
 
 
-def feed(runner, seqs, plan):
-    """plan: steps of (request, n tokens); logits of every fed token per request."""
-    got = {r: [] for r in seqs}
+def feed(runner, seqs, plan, wanted):
+    """plan: steps of (request, n tokens). ``wanted[r]`` = positions of r whose logits are compared.
+    -> {r: logits at wanted[r], in order}"""
+    got = {r: {} for r in seqs}
     fed = {r: 0 for r in seqs}
     for items in plan:
-        entries = []
+        entries, marks = [], []
         for r, n in items:
             if not runner.has_request(r):
                 runner.add_request(r)
-            entries.append(StepEntry(r, seqs[r][fed[r]:fed[r] + n], list(range(n))))
+            want = [p - fed[r] for p in wanted[r] if fed[r] <= p < fed[r] + n]
+            entries.append(StepEntry(r, seqs[r][fed[r]:fed[r] + n], want))
+            marks.append((r, [p for p in wanted[r] if fed[r] <= p < fed[r] + n]))
+            fed[r] += n
         out = runner.step(entries).float().cpu()
         o = 0
-        for r, n in items:
-            got[r].append(out[o:o + n])
-            o += n
-            fed[r] += n
+        for r, ps in marks:
+            for p in ps:
+                got[r][p] = out[o]
+                o += 1
+        assert o == out.shape[0]
+        for r, _ in items:
+            if fed[r] == len(seqs[r]):
+                runner.free_request(r)
+        runner.manager.check()
+    return {r: torch.stack([got[r][p] for p in wanted[r]]) for r in seqs}
+
+
+def check(w, dtype, seqs, plan, wanted):
+    got = feed(w.runners[dtype], seqs, plan, wanted)
     for r in seqs:
-        runner.free_request(r)
-    return {r: torch.cat(v) for r, v in got.items()}
+        ref = w.plain_rows(r, wanted[r])
+        err = rel_err(got[r], ref)
+        assert err < TOL[dtype], (r, dtype, err)
 
 
-def test_full_width_cuts_agree(engines):
-    V = RAW["vocab_size"]
-    seqs = {"a": random_tokens(150, V, 1), "b": random_tokens(97, V, 2), "c": random_tokens(40, V, 3)}
-    whole = [[("a", 150)], [("b", 97)], [("c", 40)]]
-    ref = feed(engines["float32"], seqs, whole)
-    got_whole = feed(engines["bfloat16"], seqs, whole)
+def every(n, step):
+    return sorted(set(range(0, n, step)) | {n - 1})
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_four_cuts_at_the_8b_widths(w8, dtype):
+    seqs = {"a": w8.seq("a", 150, 1), "b": w8.seq("b", 97, 2), "c": w8.seq("c", 40, 3)}
+    wanted = {"a": every(150, 7), "b": every(97, 5), "c": list(range(40))}
+    # whole
+    check(w8, dtype, seqs, [[("a", 150)], [("b", 97)], [("c", 40)]], wanted)
+    # most in one step, the last 32 one by one
+    one_by_one = []
+    for r, n in (("a", 150), ("b", 97), ("c", 40)):
+        one_by_one += [[(r, n - 32)]] + [[(r, 1)]] * 32
+    check(w8, dtype, seqs, one_by_one, {r: [p for p in wanted[r] if p >= len(seqs[r]) - 40] for r in seqs})
+    # portions of changing size, down to two tokens
+    check(w8, dtype, seqs, [[("a", 2)], [("a", 61)], [("a", 3)], [("a", 80)], [("a", 4)],
+                            [("b", 33)], [("b", 2)], [("b", 62)], [("c", 17)], [("c", 2)], [("c", 21)]], wanted)
+    # mixed: portions of some beside single tokens of others; blocks of finished requests are used again
     mixed = [[("a", 70), ("b", 2)], [("a", 1), ("b", 60), ("c", 17)], [("a", 65), ("b", 1), ("c", 1)],
              [("a", 1), ("b", 34), ("c", 2)]] + [[("a", 1), ("c", 1)]] * 13 + [[("c", 7)]]
-    got_mixed = feed(engines["bfloat16"], seqs, mixed)
-    for r in seqs:
-        assert rel_err(got_whole[r], ref[r]) < 3e-2, r
-        assert rel_err(got_mixed[r], ref[r]) < 3e-2, r
-        # the two cuts differ by rounding only: kernels chosen by the number of rows sum in another order
-        assert rel_err(got_mixed[r], got_whole[r]) < 2e-2, r
-    # 32-bit: cuts agree to float rounding
-    ref_mixed = feed(engines["float32"], seqs, mixed)
-    for r in seqs:
-        assert rel_err(ref_mixed[r], ref[r]) < 2e-5, r
+    check(w8, dtype, seqs, mixed, wanted)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_2048_token_prompt_whole_and_in_portions(w8, dtype):
+    """The prompt kernels at the length the bench runs them: one step of 2,048 tokens, and four portions
+    of 512 behind 300 tokens of earlier context (query tiles listed twice, keys from the cache)."""
+    n = 2348
+    seqs = {"long": w8.seq("long", n, 11)}
+    wanted = {"long": sorted({0, 1, 15, 16, 17, 299, 300, 301, 811, 812, 1023, 1024, 1323, 1324, 1836, 2047, 2048,
+                              2300, n - 2, n - 1})}
+    check(w8, dtype, seqs, [[("long", 2048)], [("long", n - 2048)]], wanted)
+    check(w8, dtype, seqs, [[("long", 300)]] + [[("long", 512)]] * 4, wanted)
+
+
+@pytest.mark.parametrize("n_req", [17, 33, 64])
+def test_many_requests_decode_together_at_the_8b_widths(w8, n_req):
+    """The decode step the bench times: 17, 33 and 64 requests, each with a context of 300 and more tokens,
+    decode together for 10 steps (bfloat16: products over K ranges whose sums the next kernel adds, the
+    q/k norm on those sums, flash decode at that batch, captured steps). Eight distinct sequences are
+    repeated over the requests: twins must agree to the bit, and all with the plain logits."""
+    distinct = {f"s{i}": w8.seq(f"s{i}", 300 + 3 * i + 10, 20 + i) for i in range(8)}
+    steps = 10
+    for dtype in ("bfloat16", "float32"):
+        if dtype == "float32" and n_req != 33:
+            continue                                   # one batch size is enough for the 32-bit path
+        runner = w8.runners[dtype]
+        rids = [f"r{j}" for j in range(n_req)]
+        src = {r: f"s{j % 8}" for j, r in enumerate(rids)}
+        for r in rids:
+            runner.add_request(r)
+        # prompts, eight requests a step
+        for lo in range(0, n_req, 8):
+            entries = [StepEntry(r, distinct[src[r]][:len(distinct[src[r]]) - steps], []) for r in rids[lo:lo + 8]]
+            runner.step(entries)
+        rows = {r: [] for r in rids}
+        for k in range(steps):
+            entries = []
+            for r in rids:
+                s = distinct[src[r]]
+                entries.append(StepEntry(r, [s[len(s) - steps + k]], [0]))
+            out = runner.step(entries).float().cpu()
+            for j, r in enumerate(rids):
+                rows[r].append(out[j])
+        for r in rids:
+            runner.free_request(r)
+        runner.manager.check()
+        for j, r in enumerate(rids):
+            s = distinct[src[r]]
+            got = torch.stack(rows[r])
+            ref = w8.plain_rows(src[r], range(len(s) - steps, len(s)))
+            err = rel_err(got, ref)
+            assert err < TOL[dtype], (r, dtype, n_req, err)
+            if j >= 8:
+                assert torch.equal(got, torch.stack(rows[rids[j % 8]])), (r, "differs from its twin in the same batch")
+
+
+@pytest.mark.parametrize("shape", ["4b", "32b"])
+def test_other_full_widths(shape):
+    """One layer of the Qwen3-4B widths (q projection wider than the model, tied head, K = 2560 and 9728: no
+    multiple of the products' 1024-wide walk) and of the Qwen3-32B widths (groups of 8 query heads,
+    feed-forward 25600): prompts whole and in portions, then 1, 8 and 20 requests decoding together."""
+    w = Width(shape, max_tokens=24 * 256, max_seqs=24)
+    try:
+        seqs = {"a": w.seq("a", 131, 1), "b": w.seq("b", 70, 2)}
+        wanted = {"a": every(131, 9), "b": every(70, 6)}
+        for dtype in ("float32", "bfloat16"):
+            check(w, dtype, seqs, [[("a", 131)], [("b", 70)]], wanted)
+            check(w, dtype, seqs, [[("a", 40), ("b", 3)], [("a", 1), ("b", 60)], [("a", 88), ("b", 1)],
+                                   [("a", 2), ("b", 6)]], wanted)
+        distinct = {f"s{i}": w.seq(f"s{i}", 90 + 5 * i, 30 + i) for i in range(4)}
+        steps = 6
+        for n_req in (1, 8, 20):
+            runner = w.runners["bfloat16"]
+            rids = [f"r{j}" for j in range(n_req)]
+            src = {r: f"s{j % 4}" for j, r in enumerate(rids)}
+            for r in rids:
+                runner.add_request(r)
+            for lo in range(0, n_req, 8):
+                runner.step([StepEntry(r, distinct[src[r]][:len(distinct[src[r]]) - steps], []) for r in rids[lo:lo + 8]])
+            rows = {r: [] for r in rids}
+            for k in range(steps):
+                out = runner.step([StepEntry(r, [distinct[src[r]][len(distinct[src[r]]) - steps + k]], [0])
+                                   for r in rids]).float().cpu()
+                for j, r in enumerate(rids):
+                    rows[r].append(out[j])
+            for r in rids:
+                runner.free_request(r)
+            for r in rids:
+                s = distinct[src[r]]
+                err = rel_err(torch.stack(rows[r]), w.plain_rows(src[r], range(len(s) - steps, len(s))))
+                assert err < TOL["bfloat16"], (shape, r, n_req, err)
+    finally:
+        del w
+        torch.cuda.empty_cache()
+
+
+def test_the_engine_hands_back_the_weights_it_was_built_from(tmp_path):
+    """``get_weight`` of a model drawn from a seed on the GPU gives the values that the same seed writes
+    into a folder on the CPU, and a model loaded from that folder hands back what the file holds."""
+    from helpers import TINY_B, make_folder, read_folder
+    from reinfer_amd.engine import LLMEngine
+    cfg = config_from_dict(TINY_B)
+    eng = LLMEngine(config=cfg, seed=1, dtype="bfloat16", num_blocks=8)
+    folder = make_folder(tmp_path, "B", "bfloat16")            # seed 1 as well
+    _, stored = read_folder(folder)
+    loaded = LLMEngine(folder, dtype="bfloat16", num_blocks=8)
+    for name in ("model.embed_tokens.weight", "model.layers.2.self_attn.k_proj.weight",
+                 "model.layers.0.post_attention_layernorm.weight", "lm_head.weight"):
+        assert torch.equal(eng.get_weight(name).float(), stored[name]), name
+        assert torch.equal(loaded.get_weight(name).float(), stored[name]), name
+    with pytest.raises(KeyError):
+        eng.get_weight("model.layers.9.mlp.up_proj.weight")
+    # the GPU draws what the CPU draws, bit for bit, also across the pieces a large tensor is drawn in
+    from reinfer_amd.weights import ParamDecl, random_tensor
+    for decl in (ParamDecl("m.weight", (5000, 4099)), ParamDecl("v.weight", (4097,), init="norm", role="vector")):
+        for dt in (torch.float32, torch.bfloat16):
+            assert torch.equal(random_tensor(decl, 3, dt, torch.device("cuda:0")).cpu(), random_tensor(decl, 3, dt)), decl.name

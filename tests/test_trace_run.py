@@ -122,3 +122,37 @@ def test_trace_run_step_by_step_over_a_pipe(tmp_path):
     finally:
         if proc.poll() is None:
             proc.kill()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_dumps_the_hidden_state_behind_every_layer(tmp_path, dtype):
+    """``--dump-layer``: a step's file holds the hidden state of its tokens behind the embedding and behind
+    every layer, in the order of the entries; against the plain implementation's, layer by layer, for a
+    portion of a prompt behind earlier context beside a single decoded token."""
+    folder = make_folder(tmp_path, "C", "bfloat16")
+    raw, weights = read_folder(folder)
+    V, h, L = raw["vocab_size"], raw["hidden_size"], raw["num_hidden_layers"]
+    seqs = {"a": random_tokens(45, V, 4), "b": random_tokens(30, V, 5)}
+    hid = {r: torch.stack(plain.hidden_states(raw, weights, t)) for r, t in seqs.items()}      # [L + 1, T, h]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": seqs["a"][:20], "want": []},
+                                {"id": "b", "tokens": seqs["b"][:29], "want": []}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": seqs["b"][29:30], "want": [0]},
+                                {"id": "a", "tokens": seqs["a"][20:45], "want": [24]}], "end": ["a", "b"]},
+    ]
+    out, dump = tmp_path / f"out_{dtype}", tmp_path / f"layers_{dtype}"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "128", "--dump-layer", str(dump)],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got0 = torch.from_numpy(np.fromfile(dump / "0.layers.f32", dtype="<f4").reshape(L + 1, 49, h))
+    got1 = torch.from_numpy(np.fromfile(dump / "1.layers.f32", dtype="<f4").reshape(L + 1, 26, h))
+    want0 = torch.cat([hid["a"][:, :20], hid["b"][:, :29]], dim=1)
+    want1 = torch.cat([hid["b"][:, 29:30], hid["a"][:, 20:45]], dim=1)
+    assert torch.equal(got0[0], want0[0].float()), "the embedding rows are copies"
+    for layer in range(1, L + 1):
+        assert rel_err(got0[layer], want0[layer]) < TOL[dtype], layer
+        assert rel_err(got1[layer], want1[layer]) < TOL[dtype], layer
+    # the logits files are what they are without the option
+    assert (out / "1.f32").exists() and not (out / "0.f32").exists()
