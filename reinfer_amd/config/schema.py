@@ -98,6 +98,10 @@ class PositionSpec:
     kind: str            # e.g. "rope_neox"; "none" for no position encoding
     rotary_dim: int = 0
     theta: float = 10000.0
+    extra: Tuple[Tuple[str, Any], ...] = ()   # for position parts defined elsewhere
+
+    def option(self, name: str, default: Any = None) -> Any:
+        return dict(self.extra).get(name, default)
 
 
 @dataclass(frozen=True)
@@ -170,6 +174,10 @@ class ModelSpec:
     head_name: str = "lm_head.weight"
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
+    # a position encoding that is added to the embeddings (learned or computed absolute positions), for
+    # architectures whose mixers do not rotate; None: positions enter in the mixers only
+    input_position: Optional[PositionSpec] = None
+    input_position_prefix: str = "model."
 
     def __post_init__(self):
         for i, e in enumerate(self.run_order):

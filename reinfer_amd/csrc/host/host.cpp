@@ -30,6 +30,7 @@
 #include <cstdint>
 #include <cstring>
 #include <deque>
+#include <limits>
 #include <memory>
 #include <string>
 #include <unordered_map>
@@ -66,6 +67,8 @@ struct BlockPool {
   std::vector<int> free_;          // back() is handed out next
   std::vector<char> held;
   long allocs = 0, frees = 0;
+  bool log_freed = false;          // a test's hook: remember which blocks came back, for poisoning them
+  std::vector<int> freed_log;
 
   explicit BlockPool(int n) : num_blocks(n) {
     if (n <= 0) throw py::value_error("a pool needs at least one block");
@@ -90,6 +93,7 @@ struct BlockPool {
     held[b] = 0;
     free_.push_back(b);
     ++frees;
+    if (log_freed) freed_log.push_back(b);
   }
   void check() const {
     std::vector<char> seen(num_blocks, 0);
@@ -308,6 +312,24 @@ struct CacheManager {
       seen[kv.second->slot] = 1;
     }
     if ((int)requests.size() + slots.num_free() != slots.num_slots) assertion("a state slot is lost");
+  }
+
+  // A hook for tests: from now on every block given back is remembered; take_freed() hands the list of
+  // each group over and forgets it. (A test fills those blocks with NaN, so that a kernel that reads a
+  // slot its request no longer holds shows.)
+  void log_freed(bool on) {
+    for (auto& p : pools) {
+      p.log_freed = on;
+      p.freed_log.clear();
+    }
+  }
+  std::vector<std::vector<int>> take_freed() {
+    std::vector<std::vector<int>> out;
+    for (auto& p : pools) {
+      out.push_back(p.freed_log);
+      p.freed_log.clear();
+    }
+    return out;
   }
 
   py::dict stats() const {
@@ -638,10 +660,13 @@ struct Scheduler {
     if (count) ++c_refused;
     raise_instance(*E_RequestRefused, (*E_RequestRefused)(why));
   }
+  // Tokens the smallest pool holds. A model none of whose layers keeps keys has no pool at all: its
+  // requests hold a state slot each and nothing that grows, so only the slots (and the context) bound it.
   int pool_tokens() const {
-    int n = manager->pools.at(0).num_blocks;
-    for (auto& p : manager->pools) n = std::min(n, p.num_blocks);
-    return n * manager->block_size;
+    if (manager->pools.empty()) return std::numeric_limits<int>::max() / 2;
+    long n = manager->pools.at(0).num_blocks;
+    for (auto& p : manager->pools) n = std::min<long>(n, p.num_blocks);
+    return (int)std::min<long>(n * manager->block_size, std::numeric_limits<int>::max() / 2);
   }
 
   RequestP add(const py::object& rid, const std::vector<int>& prompt, const py::object& params, const py::object& seed) {
@@ -1091,6 +1116,8 @@ PYBIND11_MODULE(_host, m) {
       .def("slot_of", &CacheManager::slot_of)
       .def("check", &CacheManager::check)
       .def("stats", &CacheManager::stats)
+      .def("log_freed", &CacheManager::log_freed, py::arg("on") = true)
+      .def("take_freed", &CacheManager::take_freed)
       .def("step_shape", &CacheManager::step_shape)
       .def("fill_step", &CacheManager::fill_step)
       .def("begin_step", &CacheManager::begin_step, py::arg("entries"), py::arg("vocab"), py::arg("max_model_len"))

@@ -12,7 +12,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..cache import CacheGroupSpec, CacheManager, OutOfBlocks, plan_groups
+from ..cache import CacheManager, OutOfBlocks, plan_groups
 from ..cache.layout import cache_shape
 from ..config import load_config
 from ..config.schema import ModelSpec
@@ -47,6 +47,7 @@ class ModelRunner:
         self.spec = spec
         self.dtype = dtype
         self.device = device
+        self._poison = False
         self._weight_source = ("given", weights)       # replaced by from_folder / from_config; see get_weight
         self.load_report: Dict[str, object] = {}
         self.block_size = int(block_size)
@@ -62,9 +63,9 @@ class ModelRunner:
                 windows.append(need.window)
             else:
                 windows.append(None)
+        # no layer with keys of its own: no group, no pool, no block tables; requests then hold a state
+        # slot each and are admitted by slots alone
         groups = plan_groups(windows)
-        if not groups:
-            groups = [CacheGroupSpec(window=0, entries=())]     # block tables exist even if unused
         self.groups = groups
         group_of = {i: g for g, gs in enumerate(groups) for i in gs.entries}
 
@@ -101,8 +102,14 @@ class ModelRunner:
                 self.caches.append(None)
 
         # decode steps replay captured graphs when every part says it can be captured
-        safe = all(getattr(getattr(b, "mixer", None), "graph_safe", False)
-                   and getattr(getattr(b, "ffn", None), "graph_safe", False) for b in self.model.blocks)
+        # (a block arrangement says so itself with ``graph_safe``, or it is asked of its ``mixer`` and ``ffn``)
+        def block_safe(b) -> bool:
+            if hasattr(b, "graph_safe"):
+                return bool(b.graph_safe)
+            return bool(getattr(getattr(b, "mixer", None), "graph_safe", False)
+                        and getattr(getattr(b, "ffn", None), "graph_safe", False))
+        safe = all(block_safe(b) for b in self.model.blocks) and \
+            (self.model.input_position is None or bool(getattr(self.model.input_position, "graph_safe", False)))
         if use_graphs is None:
             use_graphs = True
         self.graphs = None
@@ -193,6 +200,25 @@ class ModelRunner:
 
     def free_request(self, rid: Hashable) -> None:
         self.manager.free(rid)
+        if self._poison:
+            self._poison_freed()
+
+    def poison_freed_blocks(self, on: bool = True) -> None:
+        """A hook for tests: from now on the keys and values of every block that goes back to its pool (a
+        request ended, a window passed it) are overwritten with NaN at once, so that a kernel that reads a
+        slot its request no longer holds gives NaN instead of stale values that look right."""
+        self._poison = bool(on)
+        self.manager.log_freed(self._poison)
+
+    def _poison_freed(self) -> None:
+        for g, blocks in enumerate(self.manager.take_freed()):
+            if not blocks:
+                continue
+            idx = torch.tensor(sorted(set(blocks)), dtype=torch.long, device=self.device)
+            for cache in self.caches:
+                if cache is not None and cache.k is not None and cache.writes and cache.group == g:
+                    cache.k[idx] = float("nan")
+                    cache.v[idx] = float("nan")
 
     def has_request(self, rid: Hashable) -> bool:
         return rid in self.manager
@@ -235,6 +261,8 @@ class ModelRunner:
             batch = build_step_batch(entries, self.manager, self.device, pin=self.device.type == "cuda")
             logits = self.forward(batch, observer)
         self.manager.end_step(entries)
+        if self._poison:
+            self._poison_freed()           # blocks a window has passed
         return logits, tokens
 
     def forward(self, batch: StepBatch, observer=None) -> torch.Tensor:

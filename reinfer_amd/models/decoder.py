@@ -17,6 +17,10 @@ from ..weights import MATRIX, ParamDecl
 def declare_params(spec: ModelSpec) -> List[ParamDecl]:
     """Every tensor the model reads, each once, in a fixed order."""
     out = [ParamDecl(spec.embed_name, (spec.vocab_size, spec.hidden))]
+    if spec.input_position is not None:
+        part = lookup("position", spec.input_position.kind)
+        if hasattr(part, "declare_input_params"):
+            out += part.declare_input_params(spec.input_position, spec.input_position_prefix)
     for b in spec.blocks:
         out += lookup("block", b.kind).declare_params(b)
     out += lookup("norm", spec.final_norm.kind).declare_params(spec.final_norm, spec.final_norm_name)
@@ -37,6 +41,16 @@ class DecoderModel:
         self.dtype = dtype
         self.device = device
         self.embed = weights[spec.embed_name]
+        # a position part at the embedding stage: built with the model's tensors, it adds its encoding of
+        # the step's positions into the stream (``add_to_stream(resid, batch)``)
+        self.input_position = None
+        if spec.input_position is not None:
+            part = lookup("position", spec.input_position.kind)
+            if not hasattr(part, "add_to_stream"):
+                raise ValueError(f"position part {spec.input_position.kind!r} cannot stand at the embedding: "
+                                 "it has no add_to_stream(resid, batch)")
+            self.input_position = part(spec.input_position, device, weights=weights,
+                                       prefix=spec.input_position_prefix, dtype=dtype)
         self.blocks = [lookup("block", b.kind)(b, weights, dtype, device) for b in spec.blocks]
         self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, weights,
                                                                spec.final_norm_name, dtype, device)
@@ -62,6 +76,8 @@ class DecoderModel:
         ops = kernels.current()
         resid = torch.empty((batch.num_tokens, self.spec.hidden), dtype=torch.float32, device=self.device)
         ops.embed(self.embed, batch.token_ids, resid)
+        if self.input_position is not None:
+            self.input_position.add_to_stream(resid, batch)
         if observer is not None:
             observer(0, resid.clone())
         delta = None

@@ -85,6 +85,7 @@ def test_mixed_with_page_reuse(folders, plain_cache, which, dtype):
         if c is not None and c.k is not None:
             c.k.fill_(float("nan"))
             c.v.fill_(float("nan"))
+    runner.poison_freed_blocks()           # and again whenever a block goes back: a freed slot reads NaN, not stale values
     got = run_plan(runner, seqs, plan)
     for r, toks in seqs.items():
         assert rel_err(got[r], reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype], r
@@ -331,3 +332,72 @@ def test_context_limit_that_is_no_power_of_two(folders, plain_cache, limit, n):
     got = run_plan(runner, {"r": toks}, [[("r", first)]] + [[("r", 1)]] * 60)["r"]
     assert runner.graphs is not None and runner.graphs.replays >= 60
     assert rel_err(got, reference(folders, plain_cache, which, dtype, toks)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_more_requests_than_a_captured_step_holds(folders, plain_cache, dtype):
+    """136 requests decode together: above the largest captured batch, so the step runs kernel by kernel
+    with the prompt-sized products. Seventeen distinct sequences, each eight times: all agree with the
+    plain logits, and twins in one batch with each other."""
+    which = "B"
+    V = vocab(which)
+    distinct = [random_tokens(20 + 2 * i, V, 900 + i) for i in range(17)]
+    runner = runner_for(folders, which, dtype, max_tokens=136 * 64, max_seqs=136)
+    rids = [f"r{j}" for j in range(136)]
+    steps = 5
+    for lo in range(0, 136, 17):
+        runner_entries = []
+        for j in range(lo, lo + 17):
+            runner.add_request(rids[j])
+            s = distinct[j % 17]
+            runner_entries.append(StepEntry(rids[j], s[:len(s) - steps], []))
+        runner.step(runner_entries)
+    rows = {r: [] for r in rids}
+    for k in range(steps):
+        out = runner.step([StepEntry(r, [distinct[j % 17][len(distinct[j % 17]) - steps + k]], [0])
+                           for j, r in enumerate(rids)]).float().cpu()
+        for j, r in enumerate(rids):
+            rows[r].append(out[j])
+    assert runner.graphs is None or runner.graphs.replays == 0, "136 rows are more than a captured step holds"
+    for j, r in enumerate(rids):
+        s = distinct[j % 17]
+        got = torch.stack(rows[r])
+        assert rel_err(got, reference(folders, plain_cache, which, dtype, s)[-steps:]) < TOL[dtype], r
+        if j >= 17:
+            assert rel_err(got, torch.stack(rows[rids[j % 17]])) < 1e-6, r
+        runner.free_request(r)
+    runner.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sixteen_thousand_tokens_of_context(tmp_path, dtype):
+    """A context of 16,400 tokens: eight portions of 2,048 behind ever longer context, then single tokens
+    over more than a thousand blocks (split-KV decode with as many chunks as the chip takes, the 32768
+    bucket of the captured steps). The head norms of the first layer are sharpened so that single far
+    keys carry weight. The plain side runs in float32 here (a score matrix of 16,400 squared a head)."""
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.weights import write_model_folder
+    raw = dict(TINY["A"][0], max_position_embeddings=16500)
+    folder = str(tmp_path / "long16k")
+    write_model_folder(config_from_dict(raw), 12, folder, dtype=dtype)
+    rawr, weights = read_folder(folder)
+    weights = {k: v.clone() for k, v in weights.items()}
+    for name in ("q_norm", "k_norm"):
+        weights[f"model.layers.0.self_attn.{name}.weight"] *= 2.5
+    n = 16400
+    toks = random_tokens(n, raw["vocab_size"], 13)
+    rows = [0, 1, 2047, 2048, 8191, 8192, 12000, 16383] + list(range(16384, n))
+    ref = plain.forward(rawr, weights, toks, torch.float32, rows=rows).float()
+    runner = ModelRunner.from_config(config_from_dict(raw), dtype=dtype, weights=weights, max_tokens=16448)
+    runner.add_request("r")
+    got = []
+    for lo in range(0, 16384, 2048):
+        want = [p - lo for p in rows if lo <= p < lo + 2048]
+        out = runner.step([StepEntry("r", toks[lo:lo + 2048], want)])
+        if want:
+            got.append(out.float().cpu())
+    for p in range(16384, n):
+        got.append(runner.step([StepEntry("r", [toks[p]], [0])]).float().cpu())
+    got = torch.cat(got)
+    assert rel_err(got, ref) < TOL[dtype]
+    assert rel_err(got[-16:], ref[-16:]) < TOL[dtype]

@@ -299,6 +299,9 @@ def make_paged_case(dtype, Hq, Hkv, d, q_lens, starts, bs=16, seed=0, poison=Tru
     need = [-(-c // bs) for c in ctx]
     total = sum(need) + 3
     perm = torch.randperm(total, generator=g).tolist()          # shuffled physical blocks
+    if window > 0:
+        perm = [b for b in perm if b != 0]                      # block 0 is nobody's: it stays NaN (see below)
+        total += 1
     width = max(need)
     tables = torch.zeros(n_seqs, width, dtype=torch.int32)
     kc = torch.full((total, Hkv, bs, d), float("nan") if poison else 0.0)
@@ -306,6 +309,12 @@ def make_paged_case(dtype, Hq, Hkv, d, q_lens, starts, bs=16, seed=0, poison=Tru
     p = 0
     for i in range(n_seqs):
         for b in range(need[i]):
+            # As in the engine: a block that lies wholly below the window of the request's first query has
+            # been given back, and its table entry reads 0. Here block 0 holds NaN, so a kernel that reads
+            # a tile below the window's lower edge shows, whatever its mask then does with the score.
+            if window > 0 and (b + 1) * bs - 1 < starts[i] - window + 1:
+                tables[i, b] = 0
+                continue
             blk = perm[p]
             p += 1
             tables[i, b] = blk

@@ -77,6 +77,7 @@ def test_random_configurations_and_plans(tmp_path, seed, dtype):
             if c is not None and c.k is not None:
                 c.k.fill_(float("nan"))
                 c.v.fill_(float("nan"))
+        runner.poison_freed_blocks()       # a block that goes back (request ended, window passed) reads NaN from then on
         got = run_plan(runner, seqs, plan, ends=ends)
         assert all(p.num_free == p.num_blocks for p in runner.manager.pools)
         # bfloat16: the bound of helpers.TOL is for three layers; these have at most three
