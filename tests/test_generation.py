@@ -98,19 +98,28 @@ def test_temperature_generation_gpu(tmp_path):
 
 @pytest.mark.gpu
 def test_bfloat16_greedy_mostly_agrees_with_plain(tmp_path):
-    """bfloat16 may flip a near tie; where the plain top-2 gap is clear the tokens agree."""
+    """bfloat16 may flip a near tie; where the plain top-2 gap is clear the tokens agree. Clear: more than
+    twice the bound on a bfloat16 logit's error (helpers.TOL of the largest logit), so that no rounding
+    within the bound can change the order. Enough positions must have such a gap for the test to say
+    anything."""
+    from helpers import TOL
     folder = make_folder(tmp_path, "B", "bfloat16")
     raw, w = read_folder(folder)
-    prompt = random_tokens(20, raw["vocab_size"], 9)
-    out = engine_for(folder, "cuda:0", dtype="bfloat16", num_blocks=32).generate(
-        [prompt], SamplingParams(max_tokens=12))[0].token_ids
-    toks = list(prompt)
-    for t in out:
-        logits = plain.forward(raw, w, toks)[-1]
-        top2 = torch.topk(logits, 2).values
-        if (top2[0] - top2[1]) > 0.05 * logits.abs().max():
-            assert t == int(torch.argmax(logits))
-        toks.append(t)
+    eng = engine_for(folder, "cuda:0", dtype="bfloat16", num_blocks=64)
+    compared = 0
+    for seed in (9, 10, 11, 12):
+        prompt = random_tokens(20, raw["vocab_size"], seed)
+        out = eng.generate([prompt], SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))[0].token_ids
+        assert len(out) == 12
+        toks = list(prompt)
+        for t in out:
+            logits = plain.forward(raw, w, toks)[-1]
+            top2 = torch.topk(logits, 2).values
+            if (top2[0] - top2[1]) > 2.0 * TOL["bfloat16"] * logits.abs().max():
+                assert t == int(torch.argmax(logits))
+                compared += 1
+            toks.append(t)
+    assert compared >= 8, f"only {compared} of 48 positions had a clear gap"
 
 
 @pytest.mark.gpu
