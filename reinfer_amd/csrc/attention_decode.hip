@@ -38,34 +38,36 @@
 #include "common.h"
 #include "reinfer_hip.h"
 
-#define FD_THREADS 256
-#define FD_WAVES 4
+// Waves a workgroup: 4 where the step has (token, KV head) pairs enough to fill the chip with small
+// workgroups, 12 where it has few: a CU then has 192 KB of keys and values in flight for one work item,
+// few chunks a token are enough to keep the memory busy, and a token with one chunk needs no merge.
 
 __device__ __forceinline__ float fd_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// How one token's keys [lo, p] are cut: into at most max_chunks chunks of equal length, a multiple of
-// 128 and at least chunk_min (a power of two; but for the rounding), from the 16-key tile that holds lo. Equal chunks of
+// How one token's keys [lo, p] are cut: into at most max_chunks chunks of equal length, a whole number of
+// the workgroup's rounds and at least chunk_min (a power of two; but for the rounding), from the 16-key tile that holds lo. Equal chunks of
 // the token's own length, not of the longest context in the batch: no work item is a short remainder.
 struct FdCut {
   int base;    // first key of chunk 0 (a multiple of 16)
   int chunk;   // keys of a chunk
   int n;       // chunks
 };
-__device__ __forceinline__ FdCut fd_cut(int p, int lo, int chunk_shift, int max_chunks) {
+// gran: keys a workgroup takes a round (its waves x 32); a chunk is a whole number of rounds
+__device__ __forceinline__ FdCut fd_cut(int p, int lo, int chunk_shift, int max_chunks, int gran) {
   FdCut c;
   c.base = lo & ~15;
   const int span = p - c.base + 1;
   int want = (span + (1 << chunk_shift) - 1) >> chunk_shift;       // chunk_min = 1 << chunk_shift
   want = want < max_chunks ? want : max_chunks;
-  c.chunk = ((span + want - 1) / want + 127) & ~127;
-  c.n = want;                                                      // fewer if the rounding up to 128 covers the keys sooner
+  c.chunk = ((span + want - 1) / want + gran - 1) / gran * gran;
+  c.n = want;                                                      // fewer if the rounding up covers the keys sooner
   while ((c.n - 1) * c.chunk >= span) --c.n;
   return c;
 }
 
 // EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
-template <int DMAX, bool EXACT>
-__global__ void __launch_bounds__(FD_THREADS, DMAX <= 128 ? 3 : 1)
+template <int DMAX, bool EXACT, int FD_WAVES>
+__global__ void __launch_bounds__(FD_WAVES * RA_WAVE, (DMAX <= 128 && FD_WAVES == 4) ? 3 : 1)
 flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                     const int* __restrict__ block_tables, int max_blocks,
@@ -73,6 +75,7 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
                     const int* __restrict__ positions, int block_size, int Hkv, int G, int d_arg,
                     float scale_log2, int window, int chunk_shift, int max_chunks, int n_tokens,
                     int t_base, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int FD_THREADS = FD_WAVES * RA_WAVE;
   const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
@@ -90,10 +93,11 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     const int slot = item / Hkv, kvh = item % Hkv;  // KV heads of one (token, chunk) are neighbours in memory
     const int li = slot / max_chunks, ci = slot % max_chunks;
     const int t = token_list ? token_list[li] : t_base + li;
+    // seq_of_token null: every request of the step brings one token, token t is request t
+    const int seq = seq_of_token ? seq_of_token[t] : t;
     const int p = positions[t];
-    const int seq = seq_of_token[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const FdCut cut = fd_cut(p, lo, chunk_shift, max_chunks);
+    const FdCut cut = fd_cut(p, lo, chunk_shift, max_chunks, FD_WAVES * 32);
     const int n_chunks = cut.n;
     if (ci >= n_chunks) continue;
     const int* table = block_tables + (size_t)seq * max_blocks;
@@ -116,7 +120,9 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     const int k_end = min(k_begin + cut.chunk, p + 1);
     // Block ids come through the scalar cache (the index is made uniform for the compiler) and are asked
     // for one step ahead: a vector load would queue behind the K and V loads in flight, and under load a
-    // load that the K and V loads depend on costs microseconds.
+    // load that the K and V loads depend on costs microseconds. (The table's head fetched into LDS beside
+    // the position, to save the trip that waits for the position, was measured: the barrier it needs
+    // costs what the trip did.)
     auto block_of = [&](int kt_any) -> int {
       const int kt = __builtin_amdgcn_readfirstlane(kt_any);
       return (kt <= p && kt + 15 >= lo && kt < k_end) ? table[kt / block_size] : 0;
@@ -278,7 +284,7 @@ __global__ void __launch_bounds__(RA_WAVE)
 flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                           bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
                           const int* __restrict__ positions, int Hkv, int G, int d, int window, int chunk_shift,
-                          int max_chunks, int t_base) {
+                          int max_chunks, int gran, int t_base) {
   const int head = blockIdx.x, li = blockIdx.y;
   const int lane = threadIdx.x;
   const int kvh = head / G, h = head % G;
@@ -302,7 +308,7 @@ flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restr
     }
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks).n;
+    const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks, gran).n;
     if (n_chunks == 1) return;                           // written by the first kernel
     const bool mine = lane < n_chunks;
     const float mc = mine ? mc_raw : -INFINITY, lc = mine ? lc_raw : 0.f;
@@ -330,7 +336,7 @@ flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restr
   }
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks).n;
+  const int n_chunks = fd_cut(p, lo, chunk_shift, max_chunks, gran).n;
   if (n_chunks == 1) return;                           // written by the first kernel
   float acc[4] = {0.f, 0.f, 0.f, 0.f};                 // d <= 256: up to 4 outputs a lane
   float mt = -INFINITY, lt = 0.f;
@@ -377,24 +383,29 @@ flash_decode_merge_kernel(const float* __restrict__ part_o, const float* __restr
   }
 }
 
-// Workgroups of the kernel that the current device holds at once (asked once a head-size variant and
-// LDS size; the answer of the first device stands for all: one kind of GPU in a process).
-static int fd_resident_workgroups(int variant, size_t lds) {
-  static int cached[3] = {0, 0, 0};
-  static size_t cached_lds[3] = {0, 0, 0};
-  if (cached[variant] > 0 && cached_lds[variant] == lds) return cached[variant];
+// Workgroups of the kernel that the current device holds at once (asked once a head-size variant, waves a
+// workgroup and LDS size; the answer of the first device stands for all: one kind of GPU in a process).
+static int fd_resident_workgroups(int variant, int waves, size_t lds) {
+  static int cached[3][2] = {{0, 0}, {0, 0}, {0, 0}};
+  static size_t cached_lds[3][2] = {{0, 0}, {0, 0}, {0, 0}};
+  const int wi = waves == 4 ? 0 : 1;
+  if (cached[variant][wi] > 0 && cached_lds[variant][wi] == lds) return cached[variant][wi];
   int dev = 0, cus = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
   hipError_t e = hipSuccess;
   // the exact form of a head size needs a few registers more than the other: ask for it
-  if (variant == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<64, true>, FD_THREADS, lds);
-  else if (variant == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<128, true>, FD_THREADS, lds);
-  else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<256, true>, FD_THREADS, lds);
+#define RA_FD_OCC(DM)                                                                                                  \
+  e = waves == 4 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 4>, 4 * RA_WAVE, lds) \
+                 : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, flash_decode_kernel<DM, true, 12>, 12 * RA_WAVE, lds)
+  if (variant == 0) RA_FD_OCC(64);
+  else if (variant == 1) RA_FD_OCC(128);
+  else RA_FD_OCC(256);
+#undef RA_FD_OCC
   if (e != hipSuccess || cus <= 0 || per_cu <= 0) return 0;
-  cached[variant] = cus * per_cu;
-  cached_lds[variant] = lds;
-  return cached[variant];
+  cached[variant][wi] = cus * per_cu;
+  cached_lds[variant][wi] = lds;
+  return cached[variant][wi];
 }
 
 // 1 if the kernel takes these sizes, else 0 (the caller then uses the plain kernel)
@@ -405,21 +416,21 @@ extern "C" int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_si
           block_size % 16 == 0) ? 1 : 0;
 }
 
-// Workgroups of the decode kernel that the current device holds at once for these sizes (its grid); 0 if
-// the sizes are not taken or the device cannot be asked. The caller cuts the keys so that the work items
-// fill this grid once.
-extern "C" int ra_attention_decode_slots(int Hq, int Hkv, int d) {
-  if (!ra_attention_decode_supports(Hq, Hkv, d, 16)) return 0;
-  const size_t lds = (size_t)FD_WAVES * (Hq / Hkv) * (d + 2) * sizeof(float);
+// Workgroups of the decode kernel, in its form with `waves` waves a workgroup (4 or 12), that the current
+// device holds at once for these sizes (its grid); 0 if the sizes are not taken or the device cannot be
+// asked. The caller cuts the keys so that the work items fill this grid once.
+extern "C" int ra_attention_decode_slots(int Hq, int Hkv, int d, int waves) {
+  if (!ra_attention_decode_supports(Hq, Hkv, d, 16) || (waves != 4 && waves != 12)) return 0;
+  const size_t lds = (size_t)waves * (Hq / Hkv) * (d + 2) * sizeof(float);
   if (lds > 64 * 1024) return 0;
-  return fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, lds);
+  return fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, waves, lds);
 }
 
 extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride,
                                    const void* kcache, const void* vcache, const int* block_tables,
                                    int max_blocks, const int* token_list, const int* seq_of_token,
                                    const int* positions, int n_tokens, int block_size, int Hq, int Hkv,
-                                   int d, float scale, int window, int chunk, int max_chunks,
+                                   int d, float scale, int window, int chunk, int max_chunks, int waves,
                                    float* part_o, float* part_ml, hipStream_t stream) {
   RA_CHECK(n_tokens > 0, "attention_decode: no tokens");
   RA_CHECK(ra_attention_decode_supports(Hq, Hkv, d, block_size),
@@ -427,6 +438,8 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
            Hkv, d, block_size);
   RA_CHECK(max_blocks > 0 && window >= 0, "attention_decode: bad cache geometry");
   RA_CHECK(chunk >= 128 && (chunk & (chunk - 1)) == 0, "attention_decode: chunk %d is no power of two from 128", chunk);
+  if (waves == 0) waves = 4;
+  RA_CHECK(waves == 4 || waves == 12, "attention_decode: workgroups of %d waves (4 or 12)", waves);
   const int chunk_shift = __builtin_ctz((unsigned)chunk);
   RA_CHECK(max_chunks >= 1 && max_chunks <= 65535, "attention_decode: %d chunks outside 1..65535", max_chunks);
   RA_CHECK(max_chunks == 1 || (part_o && part_ml),
@@ -436,22 +449,27 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
            "attention_decode: operands must be 16-byte aligned");
   const int G = Hq / Hkv;
   const float scale_log2 = scale * 1.4426950408889634f;
-  const size_t lds = (size_t)FD_WAVES * G * (d + 2) * sizeof(float);
+  const size_t lds = (size_t)waves * G * (d + 2) * sizeof(float);
   RA_CHECK(lds <= 64 * 1024, "attention_decode: %d heads of %d per KV head need too much LDS", G, d);
-  const int slots = fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, lds);
+  const int slots = fd_resident_workgroups(d <= 64 ? 0 : d <= 128 ? 1 : 2, waves, lds);
   RA_CHECK(slots > 0, "attention_decode: cannot size the grid (%s)", hipGetErrorString(hipGetLastError()));
   const long items_max = (long)n_tokens * Hkv * max_chunks;
   RA_CHECK(items_max < (1L << 30), "attention_decode: %ld work items in one launch", items_max);
   const int grid = (int)(items_max < slots ? items_max : slots);
-#define RA_FD_GO(DM, EX)                                                                              \
-  flash_decode_kernel<DM, EX><<<grid, FD_THREADS, lds, stream>>>(                                     \
+#define RA_FD_GO(DM, EX, WV)                                                                          \
+  flash_decode_kernel<DM, EX, WV><<<grid, WV * RA_WAVE, lds, stream>>>(                               \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, token_list, seq_of_token, positions, block_size, \
       Hkv, G, d, scale_log2, window, chunk_shift, max_chunks, n_tokens, 0, part_o, part_ml)
 #define RA_FD(DM)                                                                                     \
   do {                                                                                                \
-    if (d == DM) RA_FD_GO(DM, true);                                                                  \
-    else RA_FD_GO(DM, false);                                                                         \
+    if (waves == 4) {                                                                                 \
+      if (d == DM) RA_FD_GO(DM, true, 4);                                                             \
+      else RA_FD_GO(DM, false, 4);                                                                    \
+    } else {                                                                                          \
+      if (d == DM) RA_FD_GO(DM, true, 12);                                                            \
+      else RA_FD_GO(DM, false, 12);                                                                   \
+    }                                                                                                 \
   } while (0)
   if (d <= 64) RA_FD(64);
   else if (d <= 128) RA_FD(128);
@@ -464,7 +482,7 @@ extern "C" int ra_attention_decode(const void* q, int q_stride, void* out, int o
     dim3 mg(Hq, n_tokens);
 #define RA_FDM(AH)                                                                                          \
   flash_decode_merge_kernel<AH><<<mg, RA_WAVE, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, token_list, \
-                                                           positions, Hkv, G, d, window, chunk_shift, max_chunks, 0)
+                                                           positions, Hkv, G, d, window, chunk_shift, max_chunks, waves * 32, 0)
     if (max_chunks > FDM_AHEAD) RA_FDM(0);
     else if (d <= 64) RA_FDM(1);
     else if (d <= 128) RA_FDM(2);

@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 15
+#define RA_ABI_VERSION 16
 
 #ifdef __cplusplus
 extern "C" {
@@ -89,16 +89,17 @@ int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C,
 // block_size and d are multiples of 16.
 //
 // bfloat16 flash-decode: one query per listed token. A token's keys are cut into equal chunks of its
-// own length: at most max_chunks of them, each a multiple of 128 and about `chunk` (a power of two, 128 or
-// more) or longer. With max_chunks > 1: part_o float [n_tokens * Hkv, max_chunks, G, d], part_ml float
-// [.., 2], merged by a second kernel.
+// own length: at most max_chunks of them, each a whole number of the workgroup's rounds (waves x 32 keys) and
+// about `chunk` (a power of two, 128 or more) or longer. `waves` = waves a workgroup, 4 or 12 (0: 4): 12 where
+// the step has few (token, KV head) pairs. With max_chunks > 1: part_o float [n_tokens * Hkv, max_chunks, G, d],
+// part_ml float [.., 2], merged by a second kernel.
 int ra_attention_decode_supports(int Hq, int Hkv, int d, int block_size);
-int ra_attention_decode_slots(int Hq, int Hkv, int d);   // workgroups of its grid on this device (0: unknown)
+int ra_attention_decode_slots(int Hq, int Hkv, int d, int waves);   // workgroups of its grid on this device (0: unknown)
 int ra_attention_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                         const void* vcache, const int* block_tables, int max_blocks,
                         const int* token_list, const int* seq_of_token, const int* positions,
                         int n_tokens, int block_size, int Hq, int Hkv, int d, float scale, int window,
-                        int chunk, int max_chunks, float* part_o, float* part_ml, hipStream_t stream);
+                        int chunk, int max_chunks, int waves, float* part_o, float* part_ml, hipStream_t stream);
 
 // bfloat16 flash prefill over query tiles; tile_info holds 4 ints per tile:
 // request row in block_tables, first token row, number of queries (<= tile), first position.

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 
 class KernelLibraryError(RuntimeError):
@@ -36,7 +36,7 @@ _SIGNATURES = {
     "ra_gemm_wide_partial": [P, P, P, c_long, I, I, I, I, P],
     "ra_silu_mul": [P, P, I, I, I, I, P],
     "ra_attention_plain": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, P],
-    "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P, P],
+    "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P, P],
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
@@ -75,7 +75,7 @@ def load() -> ctypes.CDLL:
             getattr(lib, name).restype = c_int
             getattr(lib, name).argtypes = [c_int, c_int, c_int, c_int]
         lib.ra_attention_decode_slots.restype = c_int
-        lib.ra_attention_decode_slots.argtypes = [c_int, c_int, c_int]
+        lib.ra_attention_decode_slots.argtypes = [c_int, c_int, c_int, c_int]
         for name in ("ra_attention_prefill_tile", "ra_attention_prefill_columns", "ra_attention_prefill_groups"):
             getattr(lib, name).restype = c_int
             getattr(lib, name).argtypes = [c_int, c_int, c_int]

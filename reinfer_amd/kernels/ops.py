@@ -375,24 +375,42 @@ class HipKernels:
                      batch.positions.data_ptr(), n, kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,
                      float(scale), int(window), _stream())
 
+    # The decode kernel runs in workgroups of 12 waves from this many (token, KV head) pairs on, or over
+    # contexts longer than this; below both, in workgroups of 4 (measured with 32 query heads over 8 KV
+    # heads of 128, flash decode and merge together: 2200 keys a token, 1 / 4 / 8 / 16 / 32 / 64 tokens: 4 waves
+    # 10.6 / 13.1 / 23.3 / 40.4 / 61.3 / 107 us, 12 waves 13.6 / 14.5 / 21.5 / 33.8 / 56.2 / 107; 8000 keys,
+    # 1 / 4 / 16 / 64 tokens: 17.9 / 35.9 / 113 / 370 against 14.7 / 31.2 / 101 / 364)
+    DECODE_WIDE_PAIRS = 64
+    DECODE_WIDE_CTX = 4096
+
     def decode_chunk(self, n_tokens: int, num_heads: int, num_kv_heads: int, head_dim: int, max_ctx: int):
-        """How the decode kernel cuts a token's keys: (least chunk length, most chunks a token).
-        The kernel cuts every token into equal chunks of its own length, so only their number is
-        chosen here: as many as fill the kernel's grid once (the workgroups the chip holds at once,
-        whatever the batch). Then all work items run side by side and the launch lasts as long as
+        """How the decode kernel cuts a token's keys: (least chunk length, most chunks a token, waves a
+        workgroup). The kernel cuts every token into equal chunks of its own length, so only their
+        number is chosen here: as many as fill the kernel's grid once (the workgroups the chip holds at
+        once, whatever the batch). Then all work items run side by side and the launch lasts as long as
         one of them; more items than that cost a start and a partial result each (measured at 2200
-        and 8000 keys a token, 1 to 128 tokens). A chunk has at least 256 keys."""
-        key = (num_heads, num_kv_heads, head_dim)
+        and 8000 keys a token, 1 to 128 tokens). Workgroups of 12 waves, one a CU, each with three times
+        the keys in flight, need a third of the chunks to keep the memory as busy, which leaves fewer
+        partial results to merge (none at 32 tokens and more); only a small step over short contexts
+        has too little work for them."""
+        pairs = max(1, n_tokens * num_kv_heads)
+        waves = 12 if (pairs >= self.DECODE_WIDE_PAIRS or max_ctx > self.DECODE_WIDE_CTX) else 4
+        key = (num_heads, num_kv_heads, head_dim, waves)
         slots = self._decode_slots.get(key)
         if slots is None:
-            slots = int(library.load().ra_attention_decode_slots(num_heads, num_kv_heads, head_dim)) or 768
+            slots = int(library.load().ra_attention_decode_slots(num_heads, num_kv_heads, head_dim, waves))
+            if slots <= 0 and waves == 12:
+                waves = 4
+                key = (num_heads, num_kv_heads, head_dim, waves)
+                slots = int(library.load().ra_attention_decode_slots(num_heads, num_kv_heads, head_dim, waves))
+            slots = slots or 768
             self._decode_slots[key] = slots
-        pairs = max(1, n_tokens * num_kv_heads)
-        return 256, max(1, min(slots // pairs, -(-max_ctx // 256)))
+        least = 256 if waves == 4 else 512
+        return least, max(1, min(slots // pairs, -(-max_ctx // least))), waves
 
     def attention_decode(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                          scale, window, group, token_list=None, n_listed=None, max_ctx=None,
-                         chunk=None) -> None:
+                         chunk=None, waves=None) -> None:
         tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, group)
         if q.dtype != torch.bfloat16:
@@ -400,8 +418,9 @@ class HipKernels:
         n = batch.num_tokens if token_list is None else int(n_listed)
         max_ctx = int(max_ctx or batch.max_ctx_len)
         if chunk is None:
-            chunk, max_chunks = self.decode_chunk(n, num_heads, num_kv_heads, head_dim, max_ctx)
+            chunk, max_chunks, waves = self.decode_chunk(n, num_heads, num_kv_heads, head_dim, max_ctx)
         else:
+            waves = int(waves or 4)
             max_chunks = max(1, -(-max_ctx // int(chunk)))
         part_o = part_ml = None
         if max_chunks > 1:
@@ -409,11 +428,13 @@ class HipKernels:
             G = num_heads // num_kv_heads
             part_o = torch.empty((pairs, max_chunks, G, head_dim), dtype=torch.float32, device=q.device)
             part_ml = torch.empty((pairs, max_chunks, G, 2), dtype=torch.float32, device=q.device)
+        # every request of the step brings one token: token t is request t, and the kernel need not look it up
+        one_each = token_list is None and batch.num_tokens == batch.num_seqs
         library.call("ra_attention_decode", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
-                     _ptr(token_list), batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), n,
+                     _ptr(token_list), None if one_each else batch.seq_of_token.data_ptr(), batch.positions.data_ptr(), n,
                      kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim, float(scale), int(window),
-                     int(chunk), int(max_chunks), _ptr(part_o), _ptr(part_ml), _stream())
+                     int(chunk), int(max_chunks), int(waves), _ptr(part_o), _ptr(part_ml), _stream())
 
     def attention_prefill(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
                           scale, window, group, tiles, n_tiles) -> None:

@@ -677,14 +677,15 @@ DEC_BATCHES = [
 def test_attention_decode(Hq, Hkv, d):
     for bi, (q_lens, starts) in enumerate(DEC_BATCHES):
         for window in (0, 19):
-            for chunk in (None, 128, 256, 1024):
+            # (least chunk, waves a workgroup); None: what the dispatch would choose (12 waves: few pairs)
+            for chunk, waves in ((None, None), (128, 4), (256, 4), (1024, 4), (128, 12), (512, 12), (2048, 12)):
                 q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=10 + bi)
                 batch = FakeBatch(q_lens, starts, tables)
                 T = sum(q_lens)
                 out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
                 scale = 1.0 / math.sqrt(d)
                 ops().attention_decode(q.view(T, Hq * d), Hq * d, out, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0,
-                                       chunk=chunk)
+                                       chunk=chunk, waves=waves)
                 ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
                 close(out, ref, 2 ** -7)     # probabilities and values are bfloat16 products summed in float
 
