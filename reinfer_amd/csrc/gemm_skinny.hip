@@ -351,13 +351,13 @@ __global__ void __launch_bounds__(WAVES * RA_WAVE, OCC)
 gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
                         const bf16_t* __restrict__ bias, TO* __restrict__ C, int ldc, int M, int N, int K,
                         SkinnyNorm nf) {
-  constexpr int MT = 1;
+  constexpr int MT = (MROWS + 15) / 16;            // row tiles of A
   constexpr int KS = U * 32;
   constexpr int LPR = U * 4;
   constexpr int RPI = RA_WAVE / LPR;
   constexpr int NI = 16 / RPI;
   constexpr int MI = (MROWS + RPI - 1) / RPI;      // load instructions that cover the rows of A
-  static_assert(MROWS <= 16, "A is one tile of 16 rows");
+  constexpr int MZ = MT * 16 / RPI;                // load instructions that would cover every row tile
   constexpr int PITCH = KS + 8;
   constexpr int TILE = 16 * PITCH;
   constexpr int STAGE = (NT + MT) * TILE;
@@ -408,19 +408,23 @@ gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      pre.c[nt][0][i] = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) pre.c[nt][mt][i] = 0.f;
       pre.w[nt][i] = 0u;
     }
   if (EPI == EPI_ACCUM && pre.have_c) {
-    const int m = r < M ? r : M - 1;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r < M ? mt * 16 + r : M - 1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int n = (int)blockIdx.x * 16 * NT + nt * 16 + 4 * g + i;
-        n = n < N ? n : N - 1;
-        pre.c[nt][0][i] = ((const float*)C)[(size_t)m * ldc + n];
-      }
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int n = (int)blockIdx.x * 16 * NT + nt * 16 + 4 * g + i;
+          n = n < N ? n : N - 1;
+          pre.c[nt][mt][i] = ((const float*)C)[(size_t)m * ldc + n];
+        }
+    }
     if (pre.have_w) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
@@ -434,12 +438,15 @@ gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
   }
   float ss_held[MT][SS_HELD] = {};
   if (nf.in_ss) {
-    const int ss_m = r < M ? r : M - 1;
 #pragma unroll
-    for (int j = 0; j < SS_HELD; ++j) {
-      int p = wave * 4 + g + j * WAVES * 4;
-      p = p < nf.in_parts ? p : nf.in_parts - 1;
-      ss_held[0][j] = nf.in_ss[(size_t)p * M + ss_m];
+    for (int mt = 0; mt < MT; ++mt) {
+      const int ss_m = mt * 16 + r < M ? mt * 16 + r : M - 1;
+#pragma unroll
+      for (int j = 0; j < SS_HELD; ++j) {
+        int p = wave * 4 + g + j * WAVES * 4;
+        p = p < nf.in_parts ? p : nf.in_parts - 1;
+        ss_held[mt][j] = nf.in_ss[(size_t)p * M + ss_m];
+      }
     }
   }
 
@@ -477,11 +484,13 @@ gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
 
   f32x4_t acc[NT][MT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) acc[nt][0] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  // rows of the A tile that no load instruction covers stay zero
+  for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-  for (int i = MI; i < NI; ++i) *(bf16x8_t*)(my + NT * TILE + (i * RPI + lr) * PITCH + lc * 8) = zero;
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // rows of the A tiles that no load instruction covers stay zero
+#pragma unroll
+  for (int i = MI; i < MZ; ++i) *(bf16x8_t*)(my + NT * TILE + (i * RPI + lr) * PITCH + lc * 8) = zero;
 
   int c_step = 0, c_n0 = (int)blockIdx.x * 16 * NT;                 // where the products are
   for (int base = 0; base < total; base += DEPTH) {
@@ -498,18 +507,22 @@ gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
       // the tile is the wave's own: its LDS operations complete in order
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       RA_DEEP_LOAD(d);
-      bf16x8_t a[NT][U], b[U];
+      bf16x8_t a[NT][U], b[MT][U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) a[nt][u] = *(const bf16x8_t*)(my + nt * TILE + r * PITCH + u * 32 + g * 8);
-        b[u] = *(const bf16x8_t*)(my + NT * TILE + r * PITCH + u * 32 + g * 8);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          b[mt][u] = *(const bf16x8_t*)(my + (NT + mt) * TILE + r * PITCH + u * 32 + g * 8);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][u], b[u], acc[nt][0], 0, 0, 0);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][u], b[mt][u], acc[nt][mt], 0, 0, 0);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // reads done before the next run overwrites the tile
     }
     c_step += DEPTH;
@@ -523,23 +536,28 @@ gemm_skinny_deep_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __r
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            asm volatile("" : "+v"(pre.c[nt][0][i]));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(pre.c[nt][mt][i]));
             asm volatile("" : "+v"(pre.w[nt][i]));
           }
       }
       if (nf.in_ss) {
 #pragma unroll
-        for (int j = 0; j < SS_HELD; ++j) {
-          asm volatile("" : "+v"(ss_held[0][j]));
-          if (!(r < M && wave * 4 + g + j * WAVES * 4 < nf.in_parts)) ss_held[0][j] = 0.f;
-        }
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int j = 0; j < SS_HELD; ++j) {
+            asm volatile("" : "+v"(ss_held[mt][j]));
+            if (!(mt * 16 + r < M && wave * 4 + g + j * WAVES * 4 < nf.in_parts)) ss_held[mt][j] = 0.f;
+          }
       }
     } else {
       pre.have_c = pre.have_w = false;      // only the first tile's values were asked for ahead
     }
     skinny_finish<MT, NT, WAVES, EPI, TO>(acc, ss_held, pre, red, row_ss, bias, C, ldc, M, N, c_n0, nf);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) acc[nt][0] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     c_step = 0;
     c_n0 += stride_n;
   }
@@ -653,7 +671,6 @@ extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* b
   }
   if (out_x || out_ss || out_w) {
     RA_CHECK(epilogue == EPI_ACCUM, "gemm_skinny: only the accumulating epilogue emits for a norm");
-    RA_CHECK(M <= 16, "gemm_skinny: with %d rows the other product kernel emits for a norm (this one up to 16)", M);
     RA_CHECK(out_x && out_ss && out_w, "gemm_skinny: emitting needs the norm weight, the scaled copy and the partial sums");
     RA_CHECK(out_w_dtype == RA_BF16 || out_w_dtype == RA_F32, "gemm_skinny: unknown norm weight dtype tag %d", out_w_dtype);
     RA_CHECK(out_ldx >= N, "gemm_skinny: the scaled copy's row stride (%d) is below %d", out_ldx, N);
@@ -669,6 +686,14 @@ extern "C" int ra_gemm_skinny_normed(const void* A, const void* W, const void* b
   if (M <= 8 && small) return launch_deep_rows<8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, stream);
   if (M <= 16 && small) return launch_deep_rows<16>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, stream);
   if (M <= 16) return launch_skinny<1, 1, 8, 4>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, stream);
+  if (small && skinny_features(M, N) == 16) {
+    // 17..64 rows, 16 features a workgroup: one workgroup a CU, runs of 64 k
+    const int n_tiles = (N + 15) / 16, cus = skinny_cus();
+    const int grid = n_tiles < cus ? n_tiles : cus;
+    if (M <= 32) return launch_deep<1, 8, 2, 2, 1, 32>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, grid, stream);
+    if (M <= 48) return launch_deep<1, 8, 2, 2, 1, 48>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, grid, stream);
+    return launch_deep<1, 8, 2, 2, 1, 64>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, grid, stream);
+  }
   if (M <= 32) return launch_skinny<2, 1, 8, 4>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, nf, stream);
   // 33..64 rows: with few output features, 16 a workgroup keep all CUs busy; with many, 32 a
   // workgroup halve the activations each one re-reads (measured at N = 4096 and 24576)

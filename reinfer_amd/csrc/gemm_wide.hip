@@ -65,7 +65,7 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                  int k_per_split, WideNorm nf) {
   constexpr int RP = WV * 4;                     // rows of the A tile a pass of the whole workgroup loads
   constexpr int AP = (MT * 16 + RP - 1) / RP;
-  constexpr int ATILE = MT * 16 * GW_PITCH;
+  constexpr int ATILE = (MT * 16 + 1) * GW_PITCH;   // one row more: where loads of rows past the tile are put
   constexpr int WTILE = 16 * GW_PITCH;
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2 * ATILE];
   __shared__ __attribute__((aligned(16))) bf16_t lds_w[WV * WTILE];
@@ -79,37 +79,54 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   const int kb = blockIdx.y * k_per_split;
   const int ke = min(K, kb + k_per_split);
   const int n_runs = (ke - kb + GW_KS - 1) / GW_KS;
+  const int n_runs_p = (n_runs + GW_DEPTH - 1) / GW_DEPTH * GW_DEPTH;      // padded with runs of zeros
   bf16_t* my_w = lds_w + wave * WTILE;
 
-  const bf16_t* wp[4];
+  // Both operands are read through buffer descriptors: a load whose offset lies past the descriptor's
+  // end returns zeros and touches no memory. Rows past N or M, chunks past the K range and the padding
+  // runs are then loads like any other: no branch stands around a load, the waits count loads exactly,
+  // and a run is used while the two behind it are still on their way. The weights' descriptor starts at
+  // the workgroup's first row; both descriptors span less than 2 GiB, and an offset with its top bit set
+  // is past their end whatever is added to it (made by arithmetic, not by a choice: the compiler turns a
+  // choice between two offsets into a branch with a load in each arm).
+  constexpr unsigned NOWHERE = 0x80000000u;
+  const int nb = blockIdx.x * WV * 16;
+  const int w_rows = min(N - nb, WV * 16);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(W) + (size_t)nb * K, 0, (int)((size_t)w_rows * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t*>(A), 0, (int)(((size_t)(M - 1) * lda + K) * 2), 0x00020000);
+  unsigned w_off[4], a_off[AP];                  // byte offset of this lane's chunk at k = 0, or NOWHERE
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    int n = n0 + i * 4 + lr;
-    n = n < N ? n : N - 1;                       // rows past the end are computed and dropped
-    wp[i] = W + (size_t)n * K + kb + lc * 8;
+    const int n = wave * 16 + i * 4 + lr;        // rows past the end are zeros; their results are dropped
+    w_off[i] = n < w_rows ? (unsigned)(((size_t)n * K + lc * 8) * 2) : NOWHERE;
   }
-  const bf16_t* ap[AP];
-  bool aok[AP];
 #pragma unroll
   for (int ps = 0; ps < AP; ++ps) {
-    int m = ps * RP + ar;
-    aok[ps] = m < M && m < MT * 16;              // rows past M are zeros, not loaded
-    m = m < M ? m : M - 1;
-    ap[ps] = A + (size_t)m * lda + kb + ac * 8;
+    const int m = ps * RP + ar;
+    a_off[ps] = (m < M && m < MT * 16) ? (unsigned)(((size_t)m * lda + ac * 8) * 2) : NOWHERE;
   }
-  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // Workgroups start their walk over K at different runs (and wrap round): if all walked in step, the
   // rows read at one moment, a whole K apart from each other, would fall on few memory channels.
   const int rot = (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)n_runs);
   auto gload = [&](GwRegs<MT, WV>& R, int run) {
-    const int k = (run + rot < n_runs ? run + rot : run + rot - n_runs) * GW_KS;
-    const bool wok = kb + k + lc * 8 < ke;       // K and the split are multiples of 8: a chunk is in or out
-    const bool kok = kb + k + ac * 8 < ke;
+    // a padding run starts at the range's end: every chunk of it is out
+    const int k = kb + (run < n_runs ? (run + rot < n_runs ? run + rot : run + rot - n_runs) * GW_KS : ke - kb);
+    // K and the split are multiples of 8: a chunk is in or out as a whole; the top bit where it is out
+    const unsigned w_out = (unsigned)((ke - 1 - (k + lc * 8)) >> 31) << 31;
+    const unsigned a_out = (unsigned)((ke - 1 - (k + ac * 8)) >> 31) << 31;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) R.w[i] = wok ? *(const bf16x8_t*)(wp[i] + k) : zero;
+    for (int i = 0; i < 4; ++i) {
+      const unsigned off = (w_off[i] + (unsigned)k * 2u) | w_out;
+      R.w[i] = __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0, 0));
+    }
 #pragma unroll
-    for (int ps = 0; ps < AP; ++ps) R.a[ps] = (kok && aok[ps]) ? *(const bf16x8_t*)(ap[ps] + k) : zero;
+    for (int ps = 0; ps < AP; ++ps) {
+      const unsigned off = (a_off[ps] + (unsigned)k * 2u) | a_out;
+      R.a[ps] = __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, 0, 0));
+    }
   };
 
   f32x4_t acc[MT];
@@ -122,9 +139,9 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
     for (int i = 0; i < 4; ++i) *(bf16x8_t*)(my_w + (i * 4 + lr) * GW_PITCH + lc * 8) = R.w[i];
 #pragma unroll
-    for (int ps = 0; ps < AP; ++ps)
-      if (ps * RP + ar < MT * 16) *(bf16x8_t*)(abuf + (ps * RP + ar) * GW_PITCH + ac * 8) = R.a[ps];
-    if (run + GW_DEPTH < n_runs) gload(R, run + GW_DEPTH);
+    for (int ps = 0; ps < AP; ++ps)      // no branch in the loop: the waits for loads stay exact
+      *(bf16x8_t*)(abuf + min(ps * RP + ar, MT * 16) * GW_PITCH + ac * 8) = R.a[ps];
+    gload(R, run + GW_DEPTH);
     // A buffer (run & 1) was last read in run - 2; every wave has passed the barrier of run - 1
     // since, so it is free. This barrier makes the tile whole before anyone reads it.
     __syncthreads();
@@ -143,8 +160,12 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 
   GwRegs<MT, WV> R[GW_DEPTH];                       // indexed by constants only once unrolled: registers
 #pragma unroll
-  for (int d = 0; d < GW_DEPTH; ++d)
-    if (d < n_runs) gload(R[d], d);
+  for (int d = 0; d < GW_DEPTH; ++d) {
+    gload(R[d], d);
+    // the runs are asked for in the order in which they are used (left alone, the scheduler asks for the
+    // first run last, and the loop then waits for every load at its head)
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // The carried norm's partial sums of row mt*16 + r, parts g, g + 4, ... a lane: the first GW_HELD of a
   // lane are asked for here, behind the first weights, and not touched before the loop is over, so that
   // no wait for them holds up the weight stream (a producer with 16 columns a workgroup leaves 256 of
@@ -154,18 +175,28 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   if (EPI != WEPI_PARTIAL && nf.in_ss) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const int m = mt * 16 + r;
+      const int m = mt * 16 + r < M ? mt * 16 + r : M - 1;       // clamped: no branch around the load
 #pragma unroll
       for (int j = 0; j < GW_HELD; ++j) {
-        const int p = g + 4 * j;
-        held[mt][j] = (m < M && p < nf.in_parts) ? nf.in_ss[(size_t)p * M + m] : 0.f;
+        const int p = g + 4 * j < nf.in_parts ? g + 4 * j : nf.in_parts - 1;
+        held[mt][j] = nf.in_ss[(size_t)p * M + m];
       }
     }
   }
-  for (int run = 0; run < n_runs; run += GW_DEPTH) {  // n_runs is the same in every thread of the workgroup
+  for (int run = 0; run < n_runs_p; run += GW_DEPTH) {  // the same in every thread of the workgroup
 #pragma unroll
-    for (int d = 0; d < GW_DEPTH; ++d)
-      if (run + d < n_runs) step(R[d], run + d);
+    for (int d = 0; d < GW_DEPTH; ++d) step(R[d], run + d);
+  }
+  if (EPI != WEPI_PARTIAL && nf.in_ss) {
+    // first touched here: an empty volatile statement per value keeps the compiler from moving
+    // arithmetic on it, and with it the wait for it, up in front of the loop
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < GW_HELD; ++j) {
+        asm volatile("" : "+v"(held[mt][j]));
+        if (!(mt * 16 + r < M && g + 4 * j < nf.in_parts)) held[mt][j] = 0.f;
+      }
   }
 
   // lane (r, g) holds C[feature n0 + 4g + i][token mt*16 + r]
@@ -187,10 +218,14 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     if (EPI == WEPI_PARTIAL) {
       if (m >= M) continue;
       float* P = (float*)C + ((size_t)blockIdx.y * M + m) * N;
+      if ((N & 3) == 0 && n0 + 4 * g + 3 < N) {
+        *(f32x4_t*)(P + n0 + 4 * g) = acc[mt];
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 4 * g + i;
-        if (n < N) P[n] = acc[mt][i];
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + 4 * g + i;
+          if (n < N) P[n] = acc[mt][i];
+        }
       }
     } else if (EPI == WEPI_ACCUM || EPI == WEPI_PLAIN) {
       if (m >= M) continue;
@@ -347,6 +382,10 @@ static int launch_wide(const void* A, int lda, const void* W, const void* bias, 
                        int epilogue, int M, int N, int K, int S, int kps, bool partial, float* scratch,
                        const WideNorm& nf, hipStream_t stream) {
   const dim3 grid((N + WV * 16 - 1) / (WV * 16), S);
+  // the kernel reads through buffer descriptors that must span less than 2 GiB: the activations, and a
+  // workgroup's 16 WV rows of weights
+  RA_CHECK(((size_t)(M - 1) * lda + K) * 2 < 0x7FFFFF00ull && (size_t)WV * 16 * K * 2 < 0x7FFFFF00ull,
+           "gemm_wide: rows of %d (stride %d) are too long for this kernel", K, lda);
 #define RA_GW(EPI, TO, OUT, LD)                                                                 \
   gemm_wide_kernel<MT, WV, EPI, TO><<<grid, WV * RA_WAVE, 0, stream>>>(                         \
       (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, (TO*)(OUT), LD, M, N, K, kps, nf)
