@@ -11,7 +11,8 @@ run through the engine's own loop (scheduler, step function, GPU sampler). One
 JSON line goes to standard output: ``value`` is decoded tokens a second at batch
 8; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the
 decode step against 8 TB/s by the bytes it must read (every weight once and the
-keys and values of the live requests); ``points`` holds batch 1 and batch 64;
+keys and values of the live requests); ``points`` holds batch 1 and batch 64, and three further
+sizes (batch 8 over 14,000-token contexts, an 8,192-token prompt, the Qwen3-32B shape at batch 8);
 ``kernel_ms`` the decode step's GPU time by kernel class with the bytes each class reads.
 ``--serve N`` runs a continuous-batching workload of N requests instead (the reference's replay harness
 feeds its scheduler synthetic arrivals the same way, crates/scheduler/src/replay.rs:180-217).
@@ -175,6 +176,49 @@ def profile_run(engine, raw, batch: int, prompt_len: int, steps: int, seed: int,
     return out
 
 
+def further_points(args, points: dict) -> None:
+    """Three more sizes into ``points``, each with an engine of its own so that the headline's engine keeps
+    the limits it is measured with: the same shape decoding at batch 8 over 14,000-token contexts, one
+    8,192-token prompt as one step, and the Qwen3-32B shape (all 64 layers) decoding at batch 8 behind
+    2,048-token prompts. Values are tokens a second."""
+    import gc
+    import torch
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.engine import LLMEngine
+    block = 16
+    steps, warmup = max(16, args.steps // 4), min(args.warmup, 16)
+
+    def engine_for(raw, batch, prompt_len, budget):
+        prompt_steps = batch * -(-prompt_len // budget)
+        max_new = prompt_steps + warmup + steps + 16
+        ctx = -(-(max(prompt_len, budget) + max_new + 32) // 1024) * 1024
+        raw = dict(raw, max_position_embeddings=ctx)
+        blocks = batch * (-(-(prompt_len + max_new + 32) // block) + 1) + -(-(budget + 16) // block) + 8
+        eng = LLMEngine(config=config_from_dict(raw), seed=args.seed, dtype=args.dtype, block_size=block,
+                        num_blocks=blocks, max_num_seqs=batch, max_num_batched_tokens=budget, max_model_len=ctx)
+        return eng, raw, max_new
+
+    def release(eng):
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    eng, raw, max_new = engine_for(QWEN3_8B, 8, 14000, 8192)
+    pf_ms = prefill_run(eng, raw, 8192, reps=3, seed=args.seed + 11)
+    points["prefill_8192"] = round(8192 / (pf_ms * 1e-3), 1)
+    log(f"prefill 8192 tokens: {pf_ms:.2f} ms, {points['prefill_8192']:.0f} tok/s")
+    ms, ctx = decode_run(eng, raw, 8, 14000, steps, warmup, args.seed + 12, max_new)
+    points["decode_b8_ctx14000"] = round(8 / (ms * 1e-3), 1)
+    log(f"decode batch 8 over contexts of {ctx:.0f} tokens: {ms:.3f} ms a step, {points['decode_b8_ctx14000']:.0f} tok/s")
+    release(eng)
+    eng, raw, max_new = engine_for(QWEN3_32B, 8, 2048, 2048)
+    ms, ctx = decode_run(eng, raw, 8, 2048, steps, warmup, args.seed + 13, max_new)
+    points["decode_b8_32b"] = round(8 / (ms * 1e-3), 1)
+    log(f"decode batch 8, Qwen3-32B shape ({raw['num_hidden_layers']} layers), contexts of {ctx:.0f} tokens: "
+        f"{ms:.3f} ms a step, {points['decode_b8_32b']:.0f} tok/s")
+    release(eng)
+
+
 def serve_run(args, raw, shape_name: str) -> int:
     """Continuous batching: ``args.serve`` requests arrive at once, prompts uniform in [64, 4096] tokens and
     outputs uniform in [32, 512], prompts cut into portions under a 2,048-token step budget beside the
@@ -235,7 +279,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points and the further sizes")
     ap.add_argument("--no-profile", action="store_true", help="skip the per-kernel-class times of the decode step")
     ap.add_argument("--profile-steps", type=int, default=4, help="decode steps timed kernel by kernel")
     ap.add_argument("--seed", type=int, default=0)
@@ -333,6 +377,12 @@ def main() -> int:
                       for k, r in kernel_ms.items()))
 
     peaks = kernels.current().measure_peaks(engine.device)
+    if not args.no_points and args.shape == "8b" and not args.layers and args.dtype == "bfloat16":
+        import gc
+        del engine          # each further size builds an engine of its own
+        gc.collect()
+        torch.cuda.empty_cache()
+        further_points(args, points)
     log(f"measured on this GPU: a plain read {peaks['hbm_read_GBps']:.0f} GB/s, bfloat16 matrix cores "
         f"{peaks['mfma_bf16_32x32x16_TFLOPs']:.0f} TFLOP/s with 32x32x16 products, {peaks['mfma_bf16_16x16x32_TFLOPs']:.0f} with "
         f"16x16x32 (nominal: {HBM_PEAK / 1e9:.0f} GB/s, {MFMA_PEAK['bf16'] / 1e12:.0f} TFLOP/s)")
