@@ -203,6 +203,36 @@ def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm, T):
     assert torch.isnan(vc.float().cpu().permute(0, 2, 1, 3)[untouched]).all()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("Hq,Hkv,d", [(4, 2, 16), (5, 5, 128), (32, 8, 128), (2, 1, 256), (6, 3, 64)])
+def test_qk_norm_rope_cache_values_of_four_slots_in_a_row(dtype, Hq, Hkv, d):
+    """A prompt's tokens sit in slots that follow each other: where four tokens in a row fill slots 4k .. 4k + 3
+    the per-token kernel writes their values in one piece. Runs of slots that start at a multiple of 4, one that
+    starts beside it, one with a token that stores nothing inside a group of four, and a ragged end."""
+    T, bs = 203, 16
+    nblk = 40
+    torch.manual_seed(d)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * d, device=DEV).to(DT[dtype])
+    src = qkv.clone()
+    slots_l = [32 + t for t in range(80)] + [321 + t for t in range(40)] + [480 + t for t in range(83)]
+    slots_l[50] = -1
+    slots = torch.tensor(slots_l, dtype=torch.int32, device=DEV)
+    positions = torch.arange(T, dtype=torch.int32, device=DEV)
+    kc = torch.full((nblk, Hkv, bs // 16, 16 * d), float("nan"), device=DEV, dtype=DT[dtype])
+    vc = torch.full_like(kc, float("nan"))
+    inv_freq = (10000.0 ** (-torch.arange(0, d, 2).double() / d)).float().to(DEV)
+    ops().qk_norm_rope_cache(qkv, None, None, 1e-6, positions, inv_freq, d, 0, slots, kc, vc, Hq, Hkv, d)
+    v = src.view(T, Hq + 2 * Hkv, d)[:, Hq + Hkv:]
+    vc = unpack_v(vc, d)
+    written = torch.zeros(nblk, bs, dtype=torch.bool)
+    for t, sl in enumerate(slots_l):
+        if sl < 0:
+            continue
+        written[sl // bs, sl % bs] = True
+        assert torch.equal(vc[sl // bs, :, sl % bs, :], v[t]), t
+    assert torch.isnan(vc.float().cpu().permute(0, 2, 1, 3)[~written]).all()
+
+
 @pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [(4, 2, 16, 16, 0, True), (3, 1, 80, 32, 0, False),
                                                       (6, 3, 64, 64, 1, True), (32, 8, 128, 128, 0, True)])
 @pytest.mark.parametrize("T,S,carried", [(5, 1, False), (33, 4, True), (64, 3, True), (20, 2, False)])
