@@ -295,7 +295,11 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
               p[ks * 4 + i] = fp_exp2(fmaf(s[ks][j][i], scale_log2, -base));      // masked: exp2(-inf) = 0
         };
         probabilities();
-        const float big = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+        // the lane's sum stands for its largest value: no probability is above 2^8 unless the sum is (it is
+        // needed anyway; a sum above 2^8 of smaller values only rescales a round early)
+        float big = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) big += p[e];
         if (__any(!(big <= 256.f) || m[j] == -INFINITY)) {           // an overflowed or undefined value counts as large
           float tmax = fmaxf(fmaxf(fmaxf(s[0][j][0], s[0][j][1]), fmaxf(s[0][j][2], s[0][j][3])),
                              fmaxf(fmaxf(s[1][j][0], s[1][j][1]), fmaxf(s[1][j][2], s[1][j][3])));
@@ -316,7 +320,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         bf16x8_t pb;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          psum += p[e];
+          psum += p[e];                                  // the same sum as above where nothing was rescaled
           pb[e] = from_f32<bf16_t>(p[e]);
         }
         l[j] += psum;
