@@ -119,6 +119,9 @@ class MixerSpec:
     bias: bool = False
     position: PositionSpec = PositionSpec("none")
     extra: Tuple[Tuple[str, Any], ...] = ()   # for mixers defined elsewhere
+    # A mixer that is not attention-shaped brings a record of its own (any frozen dataclass) with the
+    # sizes and constants it needs, typed as it likes; the fields above then stay at their defaults.
+    params: Any = None
 
     def option(self, name: str, default: Any = None) -> Any:
         return dict(self.extra).get(name, default)
@@ -130,6 +133,7 @@ class FeedForwardSpec:
     hidden: int
     intermediate: int
     extra: Tuple[Tuple[str, Any], ...] = ()
+    params: Any = None              # a record of its own for a feed-forward defined elsewhere (experts, routing)
 
 
 @dataclass(frozen=True)

@@ -3,6 +3,8 @@ without a change to the framework's files: the registries, the per-request state
 slots and the run order are all it needs. The toy keeps a decayed sum of its
 inputs per request; a model alternates it with attention, runs one block twice
 and lets the second run read the first one's cache."""
+from dataclasses import dataclass
+
 import pytest
 import torch
 
@@ -19,6 +21,12 @@ from reinfer_amd.weights import ParamDecl, random_tensors
 import plain_qwen3 as plain
 
 
+@dataclass(frozen=True)
+class DecayedSumParams:
+    """The toy mixer's own typed record (MixerSpec.params): it has no heads and no head size."""
+    decay: float
+
+
 @register_mixer("toy_decayed_sum")
 class DecayedSum:
     """s <- decay * s + x_t ;  y_t = s W^T. State: one vector per request."""
@@ -29,7 +37,7 @@ class DecayedSum:
 
     def __init__(self, spec, weights, prefix, dtype, device):
         self.w = weights[prefix + "mix.weight"]
-        self.decay = float(spec.option("decay"))
+        self.decay = spec.params.decay
         self.hidden = spec.hidden
         self.dtype = dtype
 
@@ -73,7 +81,7 @@ class ToyConfig:
         attn = MixerSpec("gqa_attention", hidden=h, num_heads=r["num_attention_heads"],
                          num_kv_heads=r["num_key_value_heads"], head_dim=d, scale=d ** -0.5, qk_norm=True,
                          qk_norm_eps=r["rms_norm_eps"], position=PositionSpec("rope_neox", d, r["rope_theta"]))
-        toy = MixerSpec("toy_decayed_sum", hidden=h, extra=(("decay", r["decay"]),))
+        toy = MixerSpec("toy_decayed_sum", hidden=h, params=DecayedSumParams(decay=float(r["decay"])))
         blocks = (BlockSpec("prenorm", attn, ffn, norm, norm, "model.layers.0."),
                   BlockSpec("prenorm", toy, ffn, norm, norm, "model.layers.1.", mixer_prefix="toy."),
                   BlockSpec("prenorm", attn, ffn, norm, norm, "model.layers.2."))

@@ -14,7 +14,7 @@ from reinfer_amd.models import declare_params
 from reinfer_amd.parts import register_position
 from reinfer_amd.sampling import SamplingParams
 from reinfer_amd.weights import ParamDecl, random_tensors
-from test_toy_mixer import DecayedSum  # noqa: F401  (registers the mixer "toy_decayed_sum")
+from test_toy_mixer import DecayedSum, DecayedSumParams  # noqa: F401  (registers the mixer "toy_decayed_sum")
 
 import plain_qwen3 as plain
 
@@ -54,7 +54,7 @@ class StateOnlyConfig:
         h = r["hidden_size"]
         norm = NormSpec("rmsnorm", h, r["rms_norm_eps"])
         ffn = FeedForwardSpec("swiglu", h, r["intermediate_size"])
-        toy = MixerSpec("toy_decayed_sum", hidden=h, extra=(("decay", r["decay"]),))
+        toy = MixerSpec("toy_decayed_sum", hidden=h, params=DecayedSumParams(decay=float(r["decay"])))
         blocks = tuple(BlockSpec("prenorm", toy, ffn, norm, norm, f"model.layers.{i}.", mixer_prefix="toy.")
                        for i in range(r["num_hidden_layers"]))
         pos = PositionSpec("toy_learned_absolute", extra=(("max_positions", r["max_position_embeddings"]), ("hidden", h)))
