@@ -236,8 +236,9 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
     if (sm.parts) {
       float row = 1.f;
       if (sm.in_ss) {
-        float tsum = 0.f;
-        for (int p = 0; p < sm.in_parts; ++p) tsum += sm.in_ss[(size_t)p * gridDim.y + t];      // fixed order
+        float tsum = 0.f;                      // the lanes share the parts out: a lane's ascending, then the lanes
+        for (int p = lane; p < sm.in_parts; p += RA_WAVE) tsum += sm.in_ss[(size_t)p * gridDim.y + t];
+        tsum = wave_sum(tsum);
         row = rsqrtf(tsum * sm.in_inv_width + sm.in_eps);
       }
       const float* src = sm.parts + ((size_t)t * n_heads + head) * d;

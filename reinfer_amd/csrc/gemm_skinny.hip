@@ -150,7 +150,7 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], const floa
         }
       ss += __shfl_xor(ss, 16, RA_WAVE);
       ss += __shfl_xor(ss, 32, RA_WAVE);
-      if (g == 0 && m < M) nf.out_ss[(size_t)blockIdx.x * M + m] = ss;
+      if (g == 0 && m < M) nf.out_ss[(size_t)(n0 / (16 * NT)) * M + m] = ss;      // the tile's number: a workgroup may take several
     }
     return;
   }

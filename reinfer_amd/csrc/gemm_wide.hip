@@ -39,12 +39,6 @@ struct WideNorm {
   float* out_ss;           // [ceil(N / 1024), M] sums of squares of C_new over 1024 columns
 };
 
-__device__ __forceinline__ float gw_rstd(const WideNorm& nf, int m, int M) {
-  float t = 0.f;
-  for (int p = 0; p < nf.in_parts; ++p) t += nf.in_ss[(size_t)p * M + m];      // fixed order
-  return rsqrtf(t * nf.in_inv_width + nf.in_eps);
-}
-
 #define GW_KS 128                      // k elements of a run
 #define GW_PITCH (GW_KS + 8)           // LDS row pitch in elements: 16 bytes of padding
 #ifndef GW_DEPTH
@@ -166,11 +160,16 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     // first run last, and the loop then waits for every load at its head)
     __builtin_amdgcn_sched_barrier(0);
   }
-  // The carried norm's partial sums of row mt*16 + r, parts g, g + 4, ... a lane: the first GW_HELD of a
-  // lane are asked for here, behind the first weights, and not touched before the loop is over, so that
-  // no wait for them holds up the weight stream (a producer with 16 columns a workgroup leaves 256 of
-  // them for a width of 4096); any further ones are read after the loop.
-  constexpr int GW_HELD = MT == 1 ? 64 : (MT == 2 ? 16 : 4);
+  // The carried norm's partial sums of row mt*16 + r: the waves and their lane groups share the parts out
+  // (lane group g of wave w takes parts 4 w + g, 4 w + g + 4 WV, ...); the first GW_HELD of a lane are asked
+  // for here, behind the first weights, and not touched before the loop is over, so that no wait for them
+  // holds up the weight stream (a producer with 16 columns a workgroup leaves 256 of them for a width of
+  // 4096: 8 a lane and row tile with eight waves); any further ones are read after the loop. The waves'
+  // sums meet in LDS, in wave order.
+  constexpr int GW_HELD = MT == 1 ? 16 : 8;
+  constexpr int PSTEP = 4 * WV;
+  __shared__ float row_ss[WV][MT * 16];
+  const int p0 = 4 * wave + g;
   float held[MT][GW_HELD];
   if (EPI != WEPI_PARTIAL && nf.in_ss) {
 #pragma unroll
@@ -178,7 +177,7 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
       const int m = mt * 16 + r < M ? mt * 16 + r : M - 1;       // clamped: no branch around the load
 #pragma unroll
       for (int j = 0; j < GW_HELD; ++j) {
-        const int p = g + 4 * j < nf.in_parts ? g + 4 * j : nf.in_parts - 1;
+        const int p = p0 + PSTEP * j < nf.in_parts ? p0 + PSTEP * j : nf.in_parts - 1;
         held[mt][j] = nf.in_ss[(size_t)p * M + m];
       }
     }
@@ -195,8 +194,22 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
       for (int j = 0; j < GW_HELD; ++j) {
         asm volatile("" : "+v"(held[mt][j]));
-        if (!(mt * 16 + r < M && g + 4 * j < nf.in_parts)) held[mt][j] = 0.f;
+        if (!(mt * 16 + r < M && p0 + PSTEP * j < nf.in_parts)) held[mt][j] = 0.f;
       }
+    // a fixed order: a lane's parts ascending, the lane groups, then the waves
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+      float t = 0.f;
+#pragma unroll
+      for (int j = 0; j < GW_HELD; ++j) t += held[mt][j];
+      if (m < M)
+        for (int p = p0 + PSTEP * GW_HELD; p < nf.in_parts; p += PSTEP) t += nf.in_ss[(size_t)p * M + m];
+      t += __shfl_xor(t, 16, RA_WAVE);
+      t += __shfl_xor(t, 32, RA_WAVE);
+      if (g == 0) row_ss[wave][mt * 16 + r] = t;
+    }
+    __syncthreads();
   }
 
   // lane (r, g) holds C[feature n0 + 4g + i][token mt*16 + r]
@@ -204,13 +217,9 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     if (EPI != WEPI_PARTIAL && nf.in_ss) {               // a split product is scaled when its parts are added
-      float t = 0.f;                                     // a fixed order: a lane's parts ascending, then the lane groups
+      float t = 0.f;
 #pragma unroll
-      for (int j = 0; j < GW_HELD; ++j) t += held[mt][j];
-      if (m < M)
-        for (int p = g + 4 * GW_HELD; p < nf.in_parts; p += 4) t += nf.in_ss[(size_t)p * M + m];
-      t += __shfl_xor(t, 16, RA_WAVE);
-      t += __shfl_xor(t, 32, RA_WAVE);
+      for (int w = 0; w < WV; ++w) t += row_ss[w][mt * 16 + r];
       const float rstd = rsqrtf(t * nf.in_inv_width + nf.in_eps);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[mt][i] *= rstd;
@@ -282,7 +291,12 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
       }
     }
   }
-  const float rstd = nf.in_ss ? gw_rstd(nf, m, M) : 1.f;
+  float rstd = 1.f;
+  if (nf.in_ss) {                              // the same for every thread: the threads share the parts out
+    float t = 0.f;
+    for (int p = threadIdx.x; p < nf.in_parts; p += blockDim.x) t += nf.in_ss[(size_t)p * M + m];
+    rstd = rsqrtf(block_sum(t, red) * nf.in_inv_width + nf.in_eps);
+  }
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {

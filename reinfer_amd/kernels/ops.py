@@ -517,8 +517,9 @@ class HipKernels:
         An RMSNorm can ride on the products around it, y = rstd[m] * ((x .* w) . W^T):
         ``row_sums`` = (ss float32 [parts, M], eps, width) scales result row m by
         rsqrt(sum_p ss[p, m] / width + eps); ``emit`` = (w [N], x_out bfloat16 [M, N],
-        ss_out float32 [skinny_row_parts(M, N), M]), with ``accumulate`` only, also writes
-        bf16(out * w) and each workgroup's sums of squares of its columns of ``out``."""
+        ss_out float32 [at least skinny_row_parts(M, N), M]), with ``accumulate`` only, also writes
+        bf16(out * w) and each workgroup's sums of squares of its columns of ``out``: into the first
+        rows of ss_out, as many as the kernel that ran has workgroups a row; that number comes back."""
         M, N, K = self._check_linear(x, weight, out, bias)
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
@@ -526,8 +527,8 @@ class HipKernels:
             raise TypeError("linear_skinny: accumulation is into a float32 matrix")
         if row_sums is None and emit is None:
             self._few_rows("linear output", x, weight, bias, out, 2 if accumulate else 0, M, N, K, wide)
-            return
-        self._skinny_normed(x, weight, bias, out, 2 if accumulate else 0, M, N, K, row_sums, emit)
+            return None
+        return self._skinny_normed(x, weight, bias, out, 2 if accumulate else 0, M, N, K, row_sums, emit)
 
     # Rows up to which an RMSNorm rides on the products around it (``row_sums`` / ``emit``) rather
     # than running as a kernel of its own: all that the weight-streaming products take. Up to 16
@@ -555,11 +556,22 @@ class HipKernels:
                      _stream())
 
     def skinny_row_parts(self, M: int, N: int) -> int:
-        """Partial sums a row that ``linear_skinny(..., emit=)`` writes for an [M, N] result."""
+        """Partial sums a row that ``linear_skinny(..., emit=)`` writes for an [M, N] result at most:
+        which of the two kernels runs, and with it the number, depends on the product's K as well."""
         lib = library.load()
+        return max(int(lib.ra_gemm_skinny_row_parts(int(M), int(N))), int(lib.ra_gemm_wide_row_parts(int(N))))
+
+    def _emits_from_skinny(self, epilogue: int, M: int, N: int, K: int) -> bool:
+        """Whether an emitting product goes to the kernel whose waves split K: up to 16 rows always; up to
+        32 where the other kernel would have to cut K into ranges and add them with a second launch for a
+        small product (an output projection of 4096 x 4096 at 32 rows: 10 us against 16; the decode step of
+        32 requests 6.19 -> 6.01 ms). With more rows the step gains nothing from it (33 and 64 requests:
+        within 0.5 %), and the consumer has 16 times the partial sums to add."""
         if M <= self.NORM_SKINNY_ROWS:
-            return int(lib.ra_gemm_skinny_row_parts(int(M), int(N)))
-        return int(lib.ra_gemm_wide_row_parts(int(N)))
+            return True
+        lib = library.load()
+        return M <= 32 and not bool(lib.ra_gemm_wide_preferred(epilogue, M, N, K)) \
+            and int(lib.ra_gemm_skinny_row_parts(M, N)) * 16 == N
 
     def _skinny_normed(self, x, weight, bias, out, epilogue, M, N, K, row_sums, emit) -> None:
         ss = eps = width = None
@@ -571,34 +583,39 @@ class HipKernels:
                 raise ValueError(f"linear_skinny: row sums {tuple(ss.shape)} {ss.dtype}, expected float32 [parts, {M}]")
             parts = ss.shape[0]
         w = xo = so = None
+        parts_out = None
         if emit is not None:
             if epilogue != 2:
                 raise ValueError("linear_skinny: only an accumulating product emits for a norm")
             w, xo, so = emit
             _dev(w, xo, so)
-            need = self.skinny_row_parts(M, N)
+            lib = library.load()
+            parts_out = int(lib.ra_gemm_skinny_row_parts(M, N)) if self._emits_from_skinny(epilogue, M, N, K) \
+                else int(lib.ra_gemm_wide_row_parts(N))
             if w.shape != (N,) or not w.is_contiguous():
                 raise ValueError(f"linear_skinny: norm weight {tuple(w.shape)}, expected [{N}]")
             if xo.dtype != torch.bfloat16 or xo.shape != (M, N) or xo.stride(1) != 1:
                 raise ValueError(f"linear_skinny: scaled copy {tuple(xo.shape)} {xo.dtype}, expected bfloat16 [{M}, {N}]")
-            if so.dtype != torch.float32 or so.shape != (need, M) or not so.is_contiguous():
-                raise ValueError(f"linear_skinny: emitted sums {tuple(so.shape)}, expected float32 [{need}, {M}]")
+            if so.dtype != torch.float32 or so.dim() != 2 or so.shape[0] < parts_out or so.shape[1] != M or not so.is_contiguous():
+                raise ValueError(f"linear_skinny: emitted sums {tuple(so.shape)}, expected float32 [{parts_out} or more, {M}]")
         norm_args = (_ptr(ss), parts, float(eps or 0.0), int(width or 0), _ptr(w),
                      _tag(w, "norm weight") if w is not None else 0, _ptr(xo),
                      xo.stride(0) if xo is not None else 0, _ptr(so))
         # the gated product of a wide feed-forward goes to the other kernel at every row count; it
         # takes row sums (any number of parts) and never emits
         gated_wide = epilogue == 1 and emit is None and bool(library.load().ra_gemm_wide_preferred(epilogue, M, N, K))
-        if M <= self.NORM_SKINNY_ROWS and not gated_wide:
+        to_skinny = self._emits_from_skinny(epilogue, M, N, K) if emit is not None else M <= self.NORM_SKINNY_ROWS
+        if to_skinny and not gated_wide:
             library.call("ra_gemm_skinny_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                          _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), *norm_args,
                          _stream())
-            return
+            return parts_out
         need = int(library.load().ra_gemm_wide_scratch(epilogue, M, N, K, 1 if emit is not None else 0))
         scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
         library.call("ra_gemm_wide_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                      _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), _ptr(scratch),
                      need, *norm_args, _stream())
+        return parts_out
 
     def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
         """True if ``linear_skinny(..., accumulate=True)`` takes this product (out += x . W^T):

@@ -106,7 +106,8 @@ class GroupedQueryAttention:
         if resid is not None and can_add and can_add(attn, self.w_o):
             # x += attn . Wo^T in the epilogue, which can also prepare the norm that follows
             if emit is not None:
-                ops.linear_skinny(attn, self.w_o, resid, accumulate=True, emit=emit.emit)
+                written = ops.linear_skinny(attn, self.w_o, resid, accumulate=True, emit=emit.emit)
+                emit.ss = emit.ss[:written]          # as many partial sums a row as the kernel that ran has workgroups
                 return emit
             ops.linear_skinny(attn, self.w_o, resid, accumulate=True)
             return None

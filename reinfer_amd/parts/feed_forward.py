@@ -71,7 +71,8 @@ class SwiGLU:
         if resid is not None and can_add and can_add(act, self.w_down):
             # x += act . Wd^T in the epilogue, which can also prepare the norm that follows
             if emit is not None:
-                ops.linear_skinny(act, self.w_down, resid, accumulate=True, emit=emit.emit)
+                written = ops.linear_skinny(act, self.w_down, resid, accumulate=True, emit=emit.emit)
+                emit.ss = emit.ss[:written]          # as many partial sums a row as the kernel that ran has workgroups
                 return emit
             ops.linear_skinny(act, self.w_down, resid, accumulate=True)
             return None

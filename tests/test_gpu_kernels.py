@@ -593,7 +593,10 @@ def test_gated_linear(M, I, K, wide):
 @pytest.mark.parametrize("M,N,K,wdt", [(1, 64, 64, torch.float32), (8, 4096, 1024, torch.float32),
                                        (13, 200, 264, torch.bfloat16), (16, 96, 4096, torch.float32),
                                        (23, 1000, 512, torch.bfloat16), (40, 328, 256, torch.float32),
-                                       (64, 9000, 128, torch.bfloat16), (64, 48, 1024, torch.float32)])
+                                       (64, 9000, 128, torch.bfloat16), (64, 48, 1024, torch.float32),
+                                       (17, 4096, 4096, torch.bfloat16), (33, 4096, 1024, torch.float32),
+                                       (64, 4096, 4096, torch.bfloat16), (48, 5120, 512, torch.bfloat16),
+                                       (64, 4096, 12288, torch.bfloat16), (8, 10240, 64, torch.bfloat16)])
 def test_rmsnorm_carried_by_two_products(M, N, K, wdt):
     """stream += a . W1^T, then y = rmsnorm(stream; w, eps) . W2^T with no norm kernel: the first
     product also writes bf16(stream * w) and partial sums of squares, the second applies the
@@ -609,7 +612,9 @@ def test_rmsnorm_carried_by_two_products(M, N, K, wdt):
     xs = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
     ss = torch.full((parts, M), float("nan"), device=DEV)
     want_stream = stream.double() + a.double() @ w1.double().T
-    ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss))
+    written = ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss))
+    assert 1 <= written <= parts and torch.isnan(ss[written:]).all()      # room for either kernel's sums; one wrote its own
+    ss = ss[:written]
     close(stream, want_stream, 2 ** -8)
     close(xs, stream.double() * nw.double(), 2 ** -8)
     close(ss.sum(0), (stream.double() ** 2).sum(1), 1e-5)
@@ -631,13 +636,14 @@ def test_rmsnorm_carried_by_two_products(M, N, K, wdt):
         close(out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
 
 
-@pytest.mark.parametrize("M", [3, 16])
+@pytest.mark.parametrize("M", [3, 16, 24, 32])
 def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
-    """Up to 16 rows the product before the norm writes one partial sum per 16 columns (256 for a
-    width of 4096); a gated product wide enough to fill the chip goes to the kernel whose waves
-    share the activations at every row count, and adds them up itself."""
+    """A small product before the norm (up to 32 rows; from 17 on, one that the other kernel would have to
+    cut into K ranges) writes one partial sum per 16 columns (256 for a width of 4096); a gated product wide
+    enough to fill the chip goes to the kernel whose waves share the activations, and adds them up itself."""
     torch.manual_seed(M)
-    N, K, J, eps = 4096, 256, 12288, 1e-6      # 24576 gated features: 256 workgroups of 96, one a CU
+    N, J, eps = 4096, 12288, 1e-6              # 24576 gated features: 256 workgroups of 96, one a CU
+    K = 256 if M <= 16 else 4096               # above 16 rows the producer stays narrow only if the other would cut K
     a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w1 = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
     stream = torch.randn(M, N, device=DEV) * 3
@@ -647,7 +653,7 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
     assert parts == N // 16
     xs = torch.empty((M, N), device=DEV, dtype=torch.bfloat16)
     ss = torch.empty((parts, M), device=DEV)
-    ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss))
+    assert ops().linear_skinny(a, w1, stream, accumulate=True, emit=(nw, xs, ss)) == parts
     normed = stream.double() * torch.rsqrt((stream.double() ** 2).mean(1, keepdim=True) + eps) * nw.double()
     wg = (torch.randn(J, N, device=DEV) * 2 / math.sqrt(N)).to(torch.bfloat16)
     wu = (torch.randn(J, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
@@ -655,6 +661,7 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
     # from 9 rows on this gated product goes to the kernel whose waves share the activations, below that
     # to the one whose workgroups stay: either must take the producer's 256 partial sums a row
     assert kernels.library.load().ra_gemm_wide_preferred(1, M, 2 * J, N) == (1 if M > 8 else 0)
+    assert kernels.library.load().ra_gemm_wide_preferred(2, M, N, K) == 0
     out = torch.full((M, J), float("nan"), device=DEV, dtype=torch.bfloat16)
     ops().gated_linear(xs, w, out, row_sums=(ss, eps, N))
     g, u = normed @ wg.double().T, normed @ wu.double().T
