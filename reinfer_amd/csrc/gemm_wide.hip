@@ -15,7 +15,9 @@
 //
 // Where N gives too few workgroups of 128 features to fill the chip, K is cut into S ranges
 // (grid.y); each writes its float partial result and a second kernel adds them in range order
-// and applies the epilogue: deterministic, no atomics. Epilogues as in gemm_skinny.hip: plain
+// and applies the epilogue: deterministic, no atomics. In that form only, the kernel also takes 65 to
+// 128 rows (six or eight row tiles): a product over a long K that adds into the residual stream is
+// faster so than the library's product followed by the add. Epilogues as in gemm_skinny.hip: plain
 // (+ bias), SiLU gate over interleaved gate/up rows (S = 1 only), C += (float).
 //
 // An RMSNorm can ride on these products as on gemm_skinny's (y = rstd[m] * ((x .* w) . W^T)): the
@@ -361,9 +363,13 @@ static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int*
 // except a small product whose K has to be cut (4096 x 4096: the second launch costs more than the
 // shared activations save); from 9 rows for the gated product of a wide feed-forward.
 extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
-  if (M < 1 || M > 64) return 0;
+  if (M < 1 || M > 128) return 0;
   int waves, S, kps;
   gw_split(epilogue, M, N, K, &waves, &S, &kps);
+  // 65 to 128 rows: the library's products are as fast or faster (151936 x 4096 at 128 rows: 285 us against
+  // 400) but for a product that adds into the residual stream over a long K, which this kernel cuts into
+  // ranges (4096 x 12288 at 96 / 128 rows: 37 / 43 us against 59 / 70 for the library's product and the add)
+  if (M > 64) return (epilogue == WEPI_ACCUM && S > 1 && (long)N * K > 4096L * 4096L) ? 1 : 0;
   // from 9 to 16 rows the gated product of a wide feed-forward (up to 8 rows the other kernel, whose
   // workgroups stay and keep two runs a wave in flight, is ahead: 24576 x 4096 36 us against 37, 51200 x
   // 5120 91 to 97 against 101 to 103): one K range, enough workgroups to fill the
@@ -391,6 +397,34 @@ extern "C" long ra_gemm_wide_scratch(int epilogue, int M, int N, int K, int emit
 // Partial sums a row that an emitting product writes for the norm that follows an [M, N] result.
 extern "C" int ra_gemm_wide_row_parts(int N) { return (N + 1023) / 1024; }
 
+// the second half of a product cut into K ranges: adds them in range order and applies the epilogue
+static int launch_wide_reduce(const void* bias, void* C, int ldc, int out_dtype, int epilogue, int M, int N, int S,
+                              const float* scratch, const WideNorm& nf, hipStream_t stream) {
+  const dim3 rg((N + 1023) / 1024, M);
+#define RA_GR(EPI, TO) \
+  gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N, nf)
+  if (epilogue == WEPI_ACCUM) RA_GR(WEPI_ACCUM, float);
+  else if (out_dtype == RA_BF16) RA_GR(WEPI_PLAIN, bf16_t);
+  else RA_GR(WEPI_PLAIN, float);
+#undef RA_GR
+  RA_LAUNCH_CHECK("gemm_wide reduce");
+  return 0;
+}
+
+// 65 to 128 rows: only as K ranges and the adding kernel (six or eight row tiles, workgroups of eight waves)
+template <int MT>
+static int launch_wide_ranges(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int out_dtype,
+                              int epilogue, int M, int N, int K, int S, int kps, float* scratch, const WideNorm& nf,
+                              hipStream_t stream) {
+  RA_CHECK(((size_t)(M - 1) * lda + K) * 2 < 0x7FFFFF00ull && (size_t)128 * K * 2 < 0x7FFFFF00ull,
+           "gemm_wide: rows of %d (stride %d) are too long for this kernel", K, lda);
+  const WideNorm none = {};
+  gemm_wide_kernel<MT, 8, WEPI_PARTIAL, float><<<dim3((N + 127) / 128, S), 8 * RA_WAVE, 0, stream>>>(
+      (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, scratch, N, M, N, K, kps, none);
+  RA_LAUNCH_CHECK("gemm_wide");
+  return launch_wide_reduce(bias, C, ldc, out_dtype, epilogue, M, N, S, scratch, nf, stream);
+}
+
 template <int MT, int WV>
 static int launch_wide(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int out_dtype,
                        int epilogue, int M, int N, int K, int S, int kps, bool partial, float* scratch,
@@ -406,15 +440,7 @@ static int launch_wide(const void* A, int lda, const void* W, const void* bias, 
   if (partial) {
     RA_GW(WEPI_PARTIAL, float, scratch, N);
     RA_LAUNCH_CHECK("gemm_wide");
-    const dim3 rg((N + 1023) / 1024, M);
-#define RA_GR(EPI, TO) \
-  gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N, nf)
-    if (epilogue == WEPI_ACCUM) RA_GR(WEPI_ACCUM, float);
-    else if (out_dtype == RA_BF16) RA_GR(WEPI_PLAIN, bf16_t);
-    else RA_GR(WEPI_PLAIN, float);
-#undef RA_GR
-    RA_LAUNCH_CHECK("gemm_wide reduce");
-    return 0;
+    return launch_wide_reduce(bias, C, ldc, out_dtype, epilogue, M, N, S, scratch, nf, stream);
   }
   if (epilogue == WEPI_SILU_PAIRS) {
     if (out_dtype == RA_BF16) RA_GW(WEPI_SILU_PAIRS, bf16_t, C, ldc);
@@ -436,7 +462,7 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
                                    int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
                                    float* out_ss, hipStream_t stream) {
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
-  RA_CHECK(M <= 64, "gemm_wide: %d rows; this kernel takes at most 64", M);
+  RA_CHECK(M <= 128, "gemm_wide: %d rows; this kernel takes at most 128", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
   RA_CHECK(epilogue == WEPI_PLAIN || epilogue == WEPI_SILU_PAIRS || epilogue == WEPI_ACCUM,
            "gemm_wide: unknown epilogue %d", epilogue);
@@ -473,6 +499,12 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
   int waves, S, kps;
   bool partial;
   gw_split(epilogue, M, N, K, &waves, &S, &kps, &partial, emits);
+  if (M > 64) {
+    RA_CHECK(partial && epilogue != WEPI_SILU_PAIRS,
+             "gemm_wide: with %d rows only a product that is cut into K ranges (64 rows otherwise)", M);
+    if (M <= 96) return launch_wide_ranges<6>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, nf, stream);
+    return launch_wide_ranges<8>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, scratch, nf, stream);
+  }
 #define RA_GWW(MT, WV) launch_wide<MT, WV>(A, lda, W, bias, C, ldc, out_dtype, epilogue, M, N, K, S, kps, partial, scratch, nf, stream)
 #define RA_GWL(MT) return waves == 5 ? RA_GWW(MT, 5) : waves == 6 ? RA_GWW(MT, 6) : waves == 7 ? RA_GWW(MT, 7) : RA_GWW(MT, 8)
   if (M <= 16) RA_GWL(1);

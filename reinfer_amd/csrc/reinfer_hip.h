@@ -67,7 +67,8 @@ int ra_gemm_skinny_normed(const void* A, const void* W, const void* bias, void* 
 // bfloat16, up to 64 rows: the same product and epilogues with the activations shared by a
 // workgroup's waves; ra_gemm_wide_preferred says where it is the faster of the two (17 rows and
 // more, not the smallest products). Small N cuts K into ranges whose float partial results need
-// `ra_gemm_wide_scratch(...)` floats of scratch (0: none needed).
+// `ra_gemm_wide_scratch(...)` floats of scratch (0: none needed). A product that is cut so may have up to
+// 128 rows (ra_gemm_wide_preferred says which are worth it: adding into the stream over a long K).
 int ra_gemm_wide_ranges(int M, int N, int K);          // K ranges of ra_gemm_wide_partial's result
 int ra_gemm_wide_partial(const void* A, const void* W, float* P, long p_floats, int M, int N, int K, int lda,
                          hipStream_t stream);         // P[range][m][n] float, for a consumer that adds the ranges

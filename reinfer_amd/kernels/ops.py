@@ -620,8 +620,12 @@ class HipKernels:
     def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
         """True if ``linear_skinny(..., accumulate=True)`` takes this product (out += x . W^T):
         the residual add of an output projection then costs no kernel and no round trip."""
-        return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and x.shape[0] <= 64 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1)
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1):
+            return False
+        M, K = x.shape
+        # above 64 rows only where the kernel that cuts K into ranges beats the library's product and an add
+        return M <= 64 or bool(library.load().ra_gemm_wide_preferred(2, M, weight.shape[0], K))
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 

@@ -672,6 +672,30 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
     close(plain_out, g / (1 + torch.exp(-g)) * u, 3 * 2 ** -8)
 
 
+@pytest.mark.parametrize("M", [65, 96, 97, 128])
+def test_accumulating_product_over_k_ranges_above_64_rows(M):
+    """65 to 128 rows: a product that adds into the float stream over a long K is cut into K ranges (six or
+    eight row tiles) where that beats the library's product and an add; other products of that many rows
+    are not taken."""
+    lib = kernels.library.load()
+    N, K = 2048, 12288
+    assert lib.ra_gemm_wide_preferred(2, M, N, K) == 1
+    assert lib.ra_gemm_wide_preferred(0, M, N, K) == 0 and lib.ra_gemm_wide_preferred(2, M, 512, 1024) == 0
+    assert lib.ra_gemm_wide_preferred(2, 129, N, K) == 0
+    torch.manual_seed(M)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    stream = torch.randn(M, N, device=DEV)
+    want = stream.double() + x.double() @ w.double().T
+    assert ops().can_accumulate(x, w)
+    ops().linear_skinny(x, w, stream, accumulate=True)
+    close(stream, want, 2 ** -8)
+    small = torch.randn(512, 1024, device=DEV).to(torch.bfloat16)
+    assert not ops().can_accumulate(x[:, :1024], small)
+    with pytest.raises(kernels.KernelLibraryError, match="rows"):
+        ops().linear_skinny(x[:, :1024], small, torch.zeros(M, 512, device=DEV), accumulate=True)
+
+
 def test_linear_dispatch_refuses_nothing_silently():
     """Sizes the MFMA kernel does not take go to the plain kernel, not to a wrong result."""
     x = torch.randn(5, 100, device=DEV).to(torch.bfloat16)[:, :99]       # K = 99, odd row stride
