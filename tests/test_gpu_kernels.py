@@ -696,6 +696,25 @@ def test_accumulating_product_over_k_ranges_above_64_rows(M):
         ops().linear_skinny(x[:, :1024], small, torch.zeros(M, 512, device=DEV), accumulate=True)
 
 
+@pytest.mark.parametrize("M", [3, 12, 40])
+def test_linear_over_a_matrix_above_4_gib(M):
+    """A vocabulary of 262144 at a width of 8192 is 4.3 GB of weights: past what one 32-bit buffer offset
+    spans. The weight-streaming kernels take it (each through the form that addresses it in 64 bits or by
+    workgroup), rows at both ends of the matrix included."""
+    N, K = 262144, 8192
+    g = torch.Generator(device=DEV).manual_seed(M)
+    w = torch.empty(N, K, device=DEV, dtype=torch.bfloat16)
+    for lo in range(0, N, 32768):                      # in pieces: the float draw of the whole would be 8.6 GB
+        w[lo:lo + 32768] = (torch.randn(32768, K, device=DEV, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    x = torch.randn(M, K, device=DEV, generator=g).to(torch.bfloat16)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops().linear(x, w, out)
+    for lo in (0, 131072 - 512, N - 1024):             # first rows, rows around the 2 GiB and 4 GiB marks, last rows
+        ref = x.double() @ w[lo:lo + 1024].double().T
+        close(out[:, lo:lo + 1024], ref, 2 ** -8)
+    assert torch.isfinite(out).all()
+
+
 def test_linear_dispatch_refuses_nothing_silently():
     """Sizes the MFMA kernel does not take go to the plain kernel, not to a wrong result."""
     x = torch.randn(5, 100, device=DEV).to(torch.bfloat16)[:, :99]       # K = 99, odd row stride
