@@ -844,6 +844,47 @@ def test_attention_prefill(Hq, Hkv, d):
                 assert torch.equal(out2, out)             # the same arithmetic, column tile by column tile
 
 
+def test_attention_and_cache_write_in_a_cache_above_4_gib():
+    """K and V of one layer at 4.9 GB each (150,000 blocks of 16 slots, 8 KV heads of 128): the attention
+    kernels and the cache write address blocks at the far end of it as they do the first."""
+    Hq, Hkv, d, NB = 32, 8, 128, 150000
+    q_lens, starts = [1, 70, 1, 3], [700, 200, 15, 40]
+    q, kc, vc, tables = make_paged_case("bfloat16", Hq, Hkv, d, q_lens, starts, seed=77)
+    small_k, small_v = kt(kc), vt(vc)                      # [blocks, kv heads, 1, 16 d]
+    n_small = small_k.shape[0]
+    far = torch.tensor([NB - 1 - 997 * b for b in range(n_small)])      # spread downwards from the last block
+    far[::3] = torch.arange(1, n_small + 1)[::3] * 11                   # and a third of them near the start
+    big_k = torch.full((NB, Hkv, 1, 16 * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    big_v = torch.full((NB, Hkv, 1, 16 * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    big_k[far.to(DEV)] = small_k
+    big_v[far.to(DEV)] = small_v
+    big_tables = far[tables.long().cpu()].to(torch.int32).to(DEV)
+    batch = FakeBatch(q_lens, starts, big_tables)
+    T = sum(q_lens)
+    scale = d ** -0.5
+    ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, 0)
+    out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().attention(q.view(T, Hq * d), Hq * d, out, big_k, big_v, batch, Hq, Hkv, d, scale, 0, 0)   # decode and prefill kernels
+    close(out, ref, 2 ** -7)
+    out = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ops().attention_plain(q.view(T, Hq * d), Hq * d, out, big_k, big_v, batch, Hq, Hkv, d, scale, 0, 0)
+    close(out, ref, 2 ** -7)
+    # the cache write, few tokens (a wave a head) and many (a workgroup a token), into the last blocks
+    for n_tok in (5, 200):
+        qkv = torch.randn(n_tok, (Hq + 2 * Hkv) * d, device=DEV).to(torch.bfloat16)
+        src = qkv.clone()
+        slots = torch.arange(n_tok, dtype=torch.int32, device=DEV) + (NB - 40) * 16
+        pos = torch.arange(n_tok, dtype=torch.int32, device=DEV)
+        inv_freq = (10000.0 ** (-torch.arange(0, d, 2).double() / d)).float().to(DEV)
+        ops().qk_norm_rope_cache(qkv, None, None, 1e-6, pos, inv_freq, d, 0, slots, big_k, big_v, Hq, Hkv, d)
+        v_rows = unpack_v(big_v[NB - 40:NB - 40 + (n_tok + 15) // 16], d)          # [blocks, kv heads, slot, d]
+        got = v_rows.permute(0, 2, 1, 3).reshape(-1, Hkv, d)[:n_tok]
+        assert torch.equal(got, src.view(n_tok, Hq + 2 * Hkv, d)[:, Hq + Hkv:])
+        k_rows = unpack_k(big_k[NB - 40:NB - 40 + (n_tok + 15) // 16], d).permute(0, 2, 1, 3).reshape(-1, Hkv, d)[:n_tok]
+        k_ref = plain.rope_neox(src.view(n_tok, Hq + 2 * Hkv, d)[:, Hq:Hq + Hkv].double().cpu(), pos.cpu(), 10000.0)
+        close(k_rows, k_ref, 2 ** -7)
+
+
 def test_attention_dispatch_mixed_batch():
     """Single tokens, a short portion and long portions in one call: each token gets
     the kernel its portion calls for, and every row is written once."""
