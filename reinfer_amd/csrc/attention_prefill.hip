@@ -54,6 +54,19 @@ static FpShape fp_shape(int Hq, int Hkv, int d) {
   return s;
 }
 
+// A listed tile may be one of several parts of a query tile, each with a range of keys (split.ranges, three
+// ints a listed tile: first key, one past the last, both multiples of the round; and the part's slot, or -1
+// for a tile that is whole): a part leaves its float sums (the outputs before the division, the running
+// maximum and the sum of each column) in its slot, and a second kernel adds a tile's parts up. A portion
+// of few queries deep in a long prompt is a handful of tiles with thousands of keys each, and a 2048-token
+// prompt is one tile a CU of which the last has 32 times the keys of the first: cut by keys, the heavy
+// tiles spread over the CUs that would idle.
+struct FpSplit {
+  const int* ranges;       // [listed tiles][3], or null: every tile is whole
+  float* part_o;           // [slots][workgroups a tile][256 columns][DMAX]
+  float* part_ml;          // [slots][workgroups a tile][256 columns][2]
+};
+
 // EXACT: the head size is DMAX itself, so every test against it is decided when the kernel is compiled
 template <int DMAX, int NC, bool EXACT>
 __global__ void __launch_bounds__(FP_THREADS)
@@ -61,7 +74,8 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
                      const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                      const int* __restrict__ block_tables, int max_blocks,
                      const int* __restrict__ tile_info,      // per tile: seq, first token row, n queries, first position
-                     int block_size, int Hq, int Hkv, int d_arg, int HG, float scale_log2, int window) {
+                     int block_size, int Hq, int Hkv, int d_arg, int HG, float scale_log2, int window,
+                     FpSplit sp) {
   const int d = EXACT ? DMAX : d_arg;
   constexpr int NDT = DMAX / 32;       // 32-wide d tiles of the score product
   constexpr int NOT = DMAX / 16;       // 16-row d tiles of the output
@@ -126,7 +140,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   // keys this tile of queries can see, and this wave's share of them
   const int last_pos = pos0 + nq - 1;
   const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-  const int kt_begin = first_key / FP_KT * FP_KT;
+  int kt_begin = first_key / FP_KT * FP_KT;
+  int k_stop = last_pos;                      // the last key of this workgroup's rounds
+  int slot = -1;
+  if (sp.ranges) {
+    kt_begin = max(kt_begin, sp.ranges[tile * 3 + 0]);
+    k_stop = min(k_stop, sp.ranges[tile * 3 + 1] - 1);
+    slot = sp.ranges[tile * 3 + 2];
+  }
   const int w_q0 = (wave * NC / HG) * 16;                       // first query of the wave
   const int w_qend = ((wave * NC + NC - 1) / HG + 1) * 16;      // one past its last
   const int w_first_pos = pos0 + w_q0;
@@ -149,7 +170,7 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
       const int c = tid + u * FP_THREADS;
       const int tt = __builtin_amdgcn_readfirstlane(c / TCH), w = c % TCH;
       const int kt = k0 + tt * 16;
-      const bool live = kt <= last_pos && kt + 15 >= first_key;         // wave-uniform
+      const bool live = kt <= k_stop && kt + 15 >= first_key;           // wave-uniform
       const int ktl = live ? kt : safe_kt;
       const int blk = table[ktl >> bs_shift];
       const size_t tile_at = (((size_t)blk * Hkv + kvh) << bs_shift) * d + (size_t)((ktl & (block_size - 1)) >> 4) * 16 * d;
@@ -357,12 +378,12 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
   __builtin_amdgcn_sched_barrier(0);
   fetch(F1, kt_begin + FP_KT);
   __builtin_amdgcn_sched_barrier(0);
-  for (int k0 = kt_begin; k0 <= last_pos; k0 += 2 * FP_KT) {     // the bounds are the same in every thread
+  for (int k0 = kt_begin; k0 <= k_stop; k0 += 2 * FP_KT) {       // the bounds are the same in every thread
     stage(F0, k0, 0);
     __syncthreads();
     fetch(F0, k0 + 2 * FP_KT);
     compute(k0, 0);
-    if (k0 + FP_KT > last_pos) break;
+    if (k0 + FP_KT > k_stop) break;
     stage(F1, k0 + FP_KT, 1);
     __syncthreads();
     fetch(F1, k0 + 3 * FP_KT);
@@ -374,6 +395,19 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     float lt = l[j];
     lt += __shfl_xor(lt, 16, RA_WAVE);
     lt += __shfl_xor(lt, 32, RA_WAVE);
+    if (slot >= 0) {
+      // a part: the sums as they are, for the kernel that adds the parts (a column without a query, or one
+      // that saw none of this part's keys, leaves zeros and -inf or 0 as its maximum: both weigh nothing)
+      const size_t col = ((size_t)slot * gy + by) * (FP_WAVES * NC * 16) + (wave * NC + j) * 16 + r;
+#pragma unroll
+      for (int ot = 0; ot < NOT; ++ot)
+        if (ot * 16 < d) *(f32x4_t*)(sp.part_o + col * DMAX + ot * 16 + 4 * g) = acc[j][ot];
+      if (g == 0) {
+        sp.part_ml[col * 2] = q_live[j] ? m[j] : -INFINITY;
+        sp.part_ml[col * 2 + 1] = lt;
+      }
+      continue;
+    }
     if (!q_live[j]) continue;
     const float inv = 1.f / lt;
     const int head = kvh * G + hgrp * HG + (wave * NC + j) % HG;
@@ -387,6 +421,89 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         *(bf16x4_t*)(op + e) = o4;
       }
     }
+  }
+}
+
+// The parts of one query tile added up, in part order: a wave takes one column (query, head) of one (tile,
+// KV head, head group); everything it may read (the maxima and sums and the outputs of up to FPM_AHEAD parts)
+// is asked for at once. merge_info, four ints a tile: first token row, queries, first slot, parts.
+#define FPM_AHEAD 8
+template <int DMAX>
+__global__ void __launch_bounds__(256)
+flash_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                           bf16_t* __restrict__ out, int out_stride, const int* __restrict__ merge_info,
+                           int gy, int n_hgrp, int G, int HG, int d, int n_cols) {
+  const int lane = threadIdx.x & (RA_WAVE - 1), wave = threadIdx.x / RA_WAVE;
+  const int groups = n_cols / 4;                         // workgroups a (tile, KV head, head group): 4 columns each
+  const int col = (blockIdx.x % groups) * 4 + wave;
+  const int by = (blockIdx.x / groups) % gy, mt = blockIdx.x / groups / gy;
+  const int kvh = by / n_hgrp, hgrp = by % n_hgrp;
+  const int row0 = merge_info[mt * 4 + 0], nq = merge_info[mt * 4 + 1];
+  const int slot0 = merge_info[mt * 4 + 2], n_parts = merge_info[mt * 4 + 3];
+  constexpr int EPL = DMAX / RA_WAVE > 0 ? DMAX / RA_WAVE : 1;
+  const int c = col / 16, r = col % 16;
+  const int qi = (c / HG) * 16 + r;
+  if (qi >= nq) return;
+  const int head = kvh * G + hgrp * HG + c % HG;
+  if (n_parts > FPM_AHEAD) {                             // many parts: one after the other
+    float mx = -INFINITY;
+    for (int p = 0; p < n_parts; ++p) mx = fmaxf(mx, part_ml[(((size_t)(slot0 + p) * gy + by) * n_cols + col) * 2]);
+    float acc[EPL], lt = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
+    for (int p = 0; p < n_parts; ++p) {
+      const size_t at = ((size_t)(slot0 + p) * gy + by) * n_cols + col;
+      const float m1 = part_ml[at * 2];
+      const float w = (m1 == -INFINITY) ? 0.f : fp_exp2(m1 - mx);
+      lt += part_ml[at * 2 + 1] * w;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + i * RA_WAVE;
+        if (e < d) acc[i] += part_o[at * DMAX + e] * w;
+      }
+    }
+    const float inv = 1.f / lt;
+    bf16_t* op = out + (size_t)(row0 + qi) * out_stride + (size_t)head * d;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + i * RA_WAVE;
+      if (e < d) op[e] = from_f32<bf16_t>(acc[i] * inv);
+    }
+    return;
+  }
+  float mp[FPM_AHEAD], lp[FPM_AHEAD], v[FPM_AHEAD][EPL];
+#pragma unroll
+  for (int p = 0; p < FPM_AHEAD; ++p) {                  // parts past the last are read again and weigh nothing
+    const size_t at = ((size_t)(slot0 + min(p, n_parts - 1)) * gy + by) * n_cols + col;
+    mp[p] = part_ml[at * 2];
+    lp[p] = part_ml[at * 2 + 1];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + i * RA_WAVE;
+      v[p][i] = part_o[at * DMAX + (e < d ? e : 0)];
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int p = 0; p < FPM_AHEAD; ++p)
+    if (p < n_parts) mx = fmaxf(mx, mp[p]);
+  float acc[EPL], lt = 0.f;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int p = 0; p < FPM_AHEAD; ++p) {                  // part order: the same sum whatever ran first
+    if (p >= n_parts) continue;
+    const float w = (mp[p] == -INFINITY) ? 0.f : fp_exp2(mp[p] - mx);
+    lt += lp[p] * w;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] += v[p][i] * w;
+  }
+  const float inv = 1.f / lt;                            // every query sees at least its own key
+  bf16_t* op = out + (size_t)(row0 + qi) * out_stride + (size_t)head * d;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + i * RA_WAVE;
+    if (e < d) op[e] = from_f32<bf16_t>(acc[i] * inv);
   }
 }
 
@@ -412,10 +529,20 @@ extern "C" int ra_attention_prefill_groups(int Hq, int Hkv, int d) {
   return Hkv * ((Hq / Hkv) / fp_shape(Hq, Hkv, d).hg);
 }
 
-extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride,
-                                    const void* kcache, const void* vcache, const int* block_tables,
-                                    int max_blocks, const int* tile_info, int n_tiles, int block_size,
-                                    int Hq, int Hkv, int d, float scale, int window, hipStream_t stream) {
+// Floats of part_o and part_ml that n_slots parts need (ra_attention_prefill_split)
+extern "C" long ra_attention_prefill_part_floats(int Hq, int Hkv, int d, int n_slots, int which) {
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || d <= 0 || n_slots <= 0) return 0;
+  const FpShape sh = fp_shape(Hq, Hkv, d);
+  const long cols = (long)n_slots * Hkv * ((Hq / Hkv) / sh.hg) * FP_WAVES * sh.nc * 16;
+  const int dmax = d <= 64 ? 64 : d <= 128 ? 128 : 256;
+  return which == 0 ? cols * dmax : cols * 2;
+}
+
+static int fp_launch(const void* q, int q_stride, void* out, int out_stride,
+                     const void* kcache, const void* vcache, const int* block_tables,
+                     int max_blocks, const int* tile_info, int n_tiles, int block_size,
+                     int Hq, int Hkv, int d, float scale, int window, const FpSplit& sp, const int* merge_info,
+                     int n_merge, hipStream_t stream) {
   RA_CHECK(n_tiles > 0, "attention_prefill: no query tiles");
   RA_CHECK(ra_attention_prefill_supports(Hq, Hkv, d, block_size),
            "attention_prefill: unsupported sizes (%d query heads, %d KV heads, head size %d, block %d)", Hq,
@@ -435,7 +562,7 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
   flash_prefill_kernel<DM, NCC, EX><<<grid, FP_THREADS, 0, stream>>>(                                 \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,                    \
       (const bf16_t*)vcache, block_tables, max_blocks, tile_info, block_size, Hq, Hkv, d, sh.hg,      \
-      scale_log2, window)
+      scale_log2, window, sp)
 #define RA_FP(DM, NCC)                                                                                \
   do {                                                                                                \
     if (d == DM && DM <= 128) RA_FP_GO(DM, NCC, true); /* at 256 the exact form spills registers */   \
@@ -447,5 +574,47 @@ extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int 
 #undef RA_FP_GO
 #undef RA_FP
   RA_LAUNCH_CHECK("attention_prefill");
+  if (n_merge > 0) {
+    const int n_cols = FP_WAVES * sh.nc * 16;
+    RA_CHECK((long)n_merge * gy * (n_cols / 4) <= 0x7fffffffL, "attention_prefill: too many tiles to add up");
+#define RA_FPM(DM)                                                                                      \
+  flash_prefill_merge_kernel<DM><<<n_merge * gy * (n_cols / 4), 256, 0, stream>>>(                      \
+      sp.part_o, sp.part_ml, (bf16_t*)out, out_stride, merge_info, gy, G / sh.hg, G, sh.hg, d, n_cols)
+    if (d <= 64) RA_FPM(64);
+    else if (d <= 128) RA_FPM(128);
+    else RA_FPM(256);
+#undef RA_FPM
+    RA_LAUNCH_CHECK("attention_prefill merge");
+  }
   return 0;
+}
+
+extern "C" int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride,
+                                    const void* kcache, const void* vcache, const int* block_tables,
+                                    int max_blocks, const int* tile_info, int n_tiles, int block_size,
+                                    int Hq, int Hkv, int d, float scale, int window, hipStream_t stream) {
+  const FpSplit none = {};
+  return fp_launch(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, tile_info, n_tiles,
+                   block_size, Hq, Hkv, d, scale, window, none, nullptr, 0, stream);
+}
+
+// The same with query tiles cut by keys: `ranges` holds three ints a listed tile (first key and one past the
+// last, multiples of 64; the part's slot, or -1 for a whole tile), `merge_info` four a cut tile (first token
+// row, queries, first slot, parts: its parts hold consecutive slots in key order); part_o and part_ml as
+// ra_attention_prefill_part_floats() sizes them for the number of slots.
+extern "C" int ra_attention_prefill_split(const void* q, int q_stride, void* out, int out_stride,
+                                          const void* kcache, const void* vcache, const int* block_tables,
+                                          int max_blocks, const int* tile_info, int n_tiles, const int* ranges,
+                                          const int* merge_info, int n_merge, float* part_o, float* part_ml,
+                                          int block_size, int Hq, int Hkv, int d, float scale, int window,
+                                          hipStream_t stream) {
+  RA_CHECK(ranges && merge_info && n_merge > 0 && part_o && part_ml,
+           "attention_prefill_split: ranges, the list of cut tiles and the buffers for their parts are needed");
+  RA_CHECK(((uintptr_t)part_o % 16) == 0, "attention_prefill_split: the parts' buffer must be 16-byte aligned");
+  FpSplit sp = {};
+  sp.ranges = ranges;
+  sp.part_o = part_o;
+  sp.part_ml = part_ml;
+  return fp_launch(q, q_stride, out, out_stride, kcache, vcache, block_tables, max_blocks, tile_info, n_tiles,
+                   block_size, Hq, Hkv, d, scale, window, sp, merge_info, n_merge, stream);
 }

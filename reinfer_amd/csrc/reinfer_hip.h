@@ -5,7 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define RA_ABI_VERSION 16
+#define RA_ABI_VERSION 17
 
 #ifdef __cplusplus
 extern "C" {
@@ -115,6 +115,16 @@ int ra_attention_prefill(const void* q, int q_stride, void* out, int out_stride,
                          const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
                          int n_tiles, int block_size, int Hq, int Hkv, int d, float scale, int window,
                          hipStream_t stream);
+// The same with query tiles cut by keys: ranges = three ints a listed tile (first key, one past the last, both
+// multiples of 64; the part's slot, or -1 for a whole tile); merge_info = four ints a cut tile (first token row,
+// queries, first slot, parts: a tile's parts hold consecutive slots in key order); part_o / part_ml: floats as
+// ra_attention_prefill_part_floats(Hq, Hkv, d, slots, 0 / 1) says. A second kernel adds the parts up in order.
+long ra_attention_prefill_part_floats(int Hq, int Hkv, int d, int n_slots, int which);
+int ra_attention_prefill_split(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                               const void* vcache, const int* block_tables, int max_blocks, const int* tile_info,
+                               int n_tiles, const int* ranges, const int* merge_info, int n_merge, float* part_o,
+                               float* part_ml, int block_size, int Hq, int Hkv, int d, float scale, int window,
+                               hipStream_t stream);
 
 int ra_sample_slices(int vocab);
 int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,

@@ -15,7 +15,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against)
 
 from ..csrc import build as _build
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 
 class KernelLibraryError(RuntimeError):
@@ -38,6 +38,7 @@ _SIGNATURES = {
     "ra_attention_plain": [P, I, P, I, P, P, I, P, I, P, P, P, I, I, I, I, I, F, I, P],
     "ra_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P, P],
     "ra_attention_prefill": [P, I, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
+    "ra_attention_prefill_split": [P, I, P, I, P, P, P, I, P, I, P, P, I, P, P, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
     "ra_gemm_wide_normed": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P, I, F, I, P, I, P, I, P, P],
@@ -79,6 +80,8 @@ def load() -> ctypes.CDLL:
         for name in ("ra_attention_prefill_tile", "ra_attention_prefill_columns", "ra_attention_prefill_groups"):
             getattr(lib, name).restype = c_int
             getattr(lib, name).argtypes = [c_int, c_int, c_int]
+        lib.ra_attention_prefill_part_floats.restype = c_long
+        lib.ra_attention_prefill_part_floats.argtypes = [c_int, c_int, c_int, c_int, c_int]
         lib.ra_sample_static_max_pairs.restype = c_long
         lib.ra_sample_static_max_pairs.argtypes = []
         lib.ra_gemm_skinny_max_rows.restype = c_int

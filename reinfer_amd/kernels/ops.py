@@ -6,6 +6,7 @@ parts call these through :func:`reinfer_amd.kernels.current`.
 """
 from __future__ import annotations
 
+import heapq
 from typing import Optional
 
 import torch
@@ -219,11 +220,10 @@ class HipKernels:
                                         head_dim, scale, window, group)
         bs = kcache.shape[2] * 16
         tile = lib.ra_attention_prefill_tile(num_heads, num_kv_heads, head_dim)
-        room = 0
-        if lib.ra_attention_prefill_columns(num_heads, num_kv_heads, head_dim) == 2:
-            # query tiles that give every CU one workgroup
-            room = self._cus(q.device) // max(1, lib.ra_attention_prefill_groups(num_heads, num_kv_heads, head_dim))
-        plan = self._attention_plan(batch, q.device, tile, room)
+        # query tiles that give every CU one workgroup
+        room = self._cus(q.device) // max(1, lib.ra_attention_prefill_groups(num_heads, num_kv_heads, head_dim))
+        halves = lib.ra_attention_prefill_columns(num_heads, num_kv_heads, head_dim) == 2
+        plan = self._attention_plan(batch, q.device, tile, room, halves)
         dec_ok = bool(lib.ra_attention_decode_supports(num_heads, num_kv_heads, head_dim, bs))
         pre_ok = bool(lib.ra_attention_prefill_supports(num_heads, num_kv_heads, head_dim, bs))
         side = None
@@ -250,7 +250,9 @@ class HipKernels:
         if plan["n_tiles"]:
             if pre_ok:
                 self.attention_prefill(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
-                                       head_dim, scale, window, group, plan["tiles"], plan["n_tiles"])
+                                       head_dim, scale, window, group, plan["tiles"], plan["n_tiles"],
+                                       plan.get("ranges"), plan.get("merge"), plan.get("n_merge", 0),
+                                       plan.get("n_slots", 0))
             else:
                 self.attention_plain(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                      head_dim, scale, window, group, plan["prefill_list"], plan["n_prefill"])
@@ -269,20 +271,118 @@ class HipKernels:
             n = self._cu_count[device] = int(torch.cuda.get_device_properties(device).multi_processor_count)
         return n
 
-    def _attention_plan(self, batch, device, tile: int, room: int = 0):
-        """Which tokens go to which kernel; made once per step and query-tile size,
-        shared by the layers. ``room`` is the number of query tiles whose workgroups fill the
-        chip once. With up to 5/4 of that, the tiles with the most keys are listed twice, each
-        time with half of the heads: the prompt kernel lasts as long as its heaviest tile, and a
-        half tile that queues behind a light one still ends before a whole heavy one would. Below
-        ``room`` tiles as many as there is room for, and at least a quarter of ``room``; from
-        ``room`` to 5/4 of it 3/16 of ``room`` (measured with 32 heads of 128 over 8 groups, room
-        32: 1024 tokens 45 -> 37 us, 1792: 65 -> 61, 2048: 84 -> 71, 2304: 94 -> 83, 2560: 104 -> 96;
-        at 3072 tokens, 48 tiles, any second listing is slower)."""
+    # What the prompt kernel's plan is chosen by, in rounds of 64 keys of a whole query tile (2.1 us with 32
+    # heads of 128 over 8 groups): a tile listed with half of its heads costs 0.76 of the whole one, every
+    # listed item one round to start and end, and the kernel that adds the parts of cut tiles 3 rounds and
+    # 0.15 for each part (measured: a portion of 512 tokens behind 3584: 142 us as it is, 115 with the tiles
+    # listed twice, 57 cut by keys; 256 behind 7936: 277 / 223 / 58; a whole prompt of 2048: 83 / 69 / 83,
+    # of 1024: 43 / 35 / 40; 2048 behind 2048: 152 / 195 / 146)
+    PREFILL_ROUND = 64
+    PREFILL_HALF_HEADS = 0.76
+    PREFILL_ITEM = 1.0
+    PREFILL_MERGE = (3.0, 0.15)
+    PREFILL_PART_ROUNDS = 4     # a part of a cut tile has at least this many rounds
+    PREFILL_MAX_PARTS = 8
+
+    @staticmethod
+    def _span(costs, room: int) -> float:
+        """When the last of ``costs`` ends if ``room`` run at a time, the heaviest started first and each
+        further one where room is first free."""
+        if len(costs) <= room:
+            return max(costs)
+        costs = sorted(costs, reverse=True)
+        ends = costs[:room]
+        heapq.heapify(ends)
+        for c in costs[room:]:
+            heapq.heappush(ends, heapq.heappop(ends) + c)
+        return max(ends)
+
+    def _prefill_items(self, tiles, room: int, halves: bool):
+        """The prompt kernel's work items for ``tiles`` of (request, row, queries, position), and the list
+        for the kernel that adds the parts of tiles cut by keys: ``(items, merge, n_slots)``, an item being
+        (cost, tile, first key, one past the last key, slot or -1).
+
+        A launch lasts as long as its heaviest item while the CUs of the light ones idle: a whole prompt of
+        2048 tokens is one tile a CU, the last with 32 times the keys of the first; a portion of 512 tokens
+        deep in a long prompt is eight tiles of thousands of keys each on a chip with room for 32. Three
+        ways to list the tiles are priced by ``_span`` and the cheapest is taken. As they are. Where the
+        kernel can give a workgroup half of a tile's heads (``halves``), the tiles with the most keys
+        twice, each time with half of the heads (as many as there is room for and at
+        least a quarter of ``room``; from ``room`` to 5/4 of it 3/16 of ``room``): a half that queues behind
+        a light tile still ends before a whole heavy one would, which pays for a prompt from its start. Or,
+        while there are fewer tiles than ``room``, the heaviest cut by keys into parts, each an item whose
+        float sums a second kernel adds up; the spare room goes, one part at a time, to the tile whose
+        parts are longest. (Windows are not known here, one plan serving all layers: a part below a
+        layer's window finds nothing to do.)"""
+        R = self.PREFILL_ROUND
+        n = len(tiles)
+        rounds = [-(-(pos + q) // R) for (_, _, q, pos) in tiles]
+        whole = [(r + self.PREFILL_ITEM, tl, 0, 0, -1) for tl, r in zip(tiles, rounds)]
+        if room <= 0 or n == 0:
+            return whole, [], 0
+        best, best_span = (whole, [], 0), self._span([it[0] for it in whole], room)
+        # the heaviest twice, by heads
+        n_twice = 0
+        if not halves:
+            pass
+        elif n <= room:
+            n_twice = min(n, max(room - n, room // 4))
+        elif n <= room + room // 4:
+            n_twice = (3 * room) // 16
+        if n_twice:
+            twice = set(sorted(range(n), key=lambda k: -rounds[k])[:n_twice])
+            items = []
+            for k, (tl, r) in enumerate(zip(tiles, rounds)):
+                if k in twice:
+                    i, row, q, pos = tl
+                    c = r * self.PREFILL_HALF_HEADS + self.PREFILL_ITEM
+                    items.append((c, (i, row, q | (1 << 16), pos), 0, 0, -1))
+                    items.append((c, (i, row, q | (2 << 16), pos), 0, 0, -1))
+                else:
+                    items.append(whole[k])
+            span = self._span([it[0] for it in items], room)
+            if span < best_span:
+                best, best_span = (items, [], 0), span
+        # the heaviest cut by keys
+        if n < room:
+            parts = [1] * n
+            heap = [(-r, k) for k, r in enumerate(rounds)]
+            heapq.heapify(heap)
+            used = n
+            while used < room and heap:
+                _, k = heapq.heappop(heap)
+                if parts[k] >= self.PREFILL_MAX_PARTS or rounds[k] < self.PREFILL_PART_ROUNDS * (parts[k] + 1):
+                    continue
+                parts[k] += 1
+                used += 1
+                heapq.heappush(heap, (-rounds[k] / parts[k], k))
+            items, merge, n_slots = [], [], 0
+            for k, (tl, r) in enumerate(zip(tiles, rounds)):
+                per = -(-r // parts[k])
+                p = -(-r // per)
+                if p <= 1:
+                    items.append(whole[k])
+                    continue
+                merge.extend((tl[1], tl[2], n_slots, p))
+                for j in range(p):
+                    hi = (j + 1) * per * R if j + 1 < p else 1 << 30
+                    items.append((min(per, r - j * per) + self.PREFILL_ITEM, tl, j * per * R, hi, n_slots + j))
+                n_slots += p
+            if n_slots:
+                span = self._span([it[0] for it in items], room) + self.PREFILL_MERGE[0] \
+                    + self.PREFILL_MERGE[1] * n_slots
+                if span < best_span:
+                    best, best_span = (items, merge, n_slots), span
+        return best
+
+    def _attention_plan(self, batch, device, tile: int, room: int = 0, halves: bool = False):
+        """Which tokens go to which kernel; made once per step and query-tile size, shared by the
+        layers. ``room`` is the number of query tiles whose workgroups fill the chip once (0: the tiles
+        are listed as they are)."""
         plan = batch.extra.get("attention_plan")
         if plan is not None and plan.get("tile", tile) == tile:
             return plan
-        plan = batch.extra.get(("attention_plan", tile, room))
+        plan = batch.extra.get(("attention_plan", tile, room, halves))
         if plan is not None:
             return plan
         dec, pre, tiles = [], [], []
@@ -295,44 +395,32 @@ class HipKernels:
             else:
                 pre.extend(range(t, t + ql))
                 for q0 in range(0, ql, tile):
-                    tiles.extend((i, t + q0, min(tile, ql - q0), st + q0))
+                    tiles.append((i, t + q0, min(tile, ql - q0), st + q0))
             t += ql
-        n_tiles = len(tiles) // 4
-        if n_tiles > 1:
-            # the kernel starts the last listed tile first: list the tiles by the keys they see, so that
-            # the longest of every request start first, whatever the order of the requests
-            quads = sorted((tuple(tiles[4 * k:4 * k + 4]) for k in range(n_tiles)), key=lambda t: t[3] + t[2])
-            tiles = [v for t in quads for v in t]
-        n_twice = 0
-        if 0 < n_tiles <= room:
-            n_twice = min(n_tiles, max(room - n_tiles, room // 4))
-        elif room < n_tiles <= room + room // 4:
-            n_twice = (3 * room) // 16
-        if n_twice:
-            by_keys = sorted(range(n_tiles), key=lambda k: -(tiles[4 * k + 3] + tiles[4 * k + 2]))
-            twice = set(by_keys[:n_twice])
-            cut = []
-            for k in range(n_tiles):
-                i, row, n, pos = tiles[4 * k:4 * k + 4]
-                if k in twice:
-                    cut.extend((i, row, n | (1 << 16), pos, i, row, n | (2 << 16), pos))
-                else:
-                    cut.extend((i, row, n, pos))
-            tiles = cut
+        items, merge, n_slots = self._prefill_items(tiles, room, halves)
+        items.sort(key=lambda it: it[0])                     # the heaviest last: the kernel starts the last listed first
+        listed = [v for it in items for v in it[1]]
+        ranges = [v for it in items for v in ((it[2], it[3], it[4]) if it[4] >= 0 else (0, 1 << 30, -1))] if merge else []
         all_decode = len(dec) == batch.num_tokens
-        flat = ([] if all_decode else dec) + pre + tiles
+        flat = ([] if all_decode else dec) + pre + listed + ranges + merge
         dev = torch.tensor(flat, dtype=torch.int32).to(device, non_blocking=True) if flat else None
         n_dec_listed = 0 if all_decode else len(dec)
+        o_tiles = n_dec_listed + len(pre)
+        o_ranges = o_tiles + len(listed)
+        o_merge = o_ranges + len(ranges)
         plan = {
             "n_decode": len(dec), "decode_max_ctx": dec_max_ctx,
             "decode_list": None if all_decode or not dec else dev[:n_dec_listed],
             "n_prefill": len(pre),
-            "prefill_list": dev[n_dec_listed:n_dec_listed + len(pre)] if pre else None,
-            "n_tiles": len(tiles) // 4,
-            "tiles": dev[n_dec_listed + len(pre):] if tiles else None,
+            "prefill_list": dev[n_dec_listed:o_tiles] if pre else None,
+            "n_tiles": len(items),
+            "tiles": dev[o_tiles:o_ranges] if items else None,
+            "ranges": dev[o_ranges:o_merge] if merge else None,
+            "merge": dev[o_merge:] if merge else None,
+            "n_merge": len(merge) // 4, "n_slots": n_slots,
             "tile": tile,
         }
-        batch.extra[("attention_plan", tile, room)] = plan
+        batch.extra[("attention_plan", tile, room, halves)] = plan
         return plan
 
     @staticmethod
@@ -447,12 +535,33 @@ class HipKernels:
                      int(chunk), int(max_chunks), int(waves), _ptr(part_o), _ptr(part_ml), _stream())
 
     def attention_prefill(self, q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads, head_dim,
-                          scale, window, group, tiles, n_tiles) -> None:
+                          scale, window, group, tiles, n_tiles, ranges=None, merge=None, n_merge: int = 0,
+                          n_slots: int = 0) -> None:
+        """``tiles``: four ints a listed query tile (request row, first token row, queries, first
+        position). With ``ranges`` (three ints a listed tile: first key, one past the last, the part's
+        slot or -1) some tiles are listed in several parts by keys, and ``merge`` (four ints a cut tile:
+        first token row, queries, first slot, parts) says which to add up."""
         tables = self._check_attention(q, q_stride, out, kcache, vcache, batch, num_heads, num_kv_heads,
                                        head_dim, group)
         if q.dtype != torch.bfloat16:
             raise TypeError("attention_prefill: bfloat16 only")
         _int32(tiles, "query tiles", 4 * n_tiles)
+        if ranges is not None:
+            _int32(ranges, "key ranges", 3 * n_tiles)
+            _int32(merge, "cut tiles", 4 * n_merge)
+            if n_merge <= 0 or n_slots <= 0:
+                raise ValueError("attention_prefill: key ranges without cut tiles")
+            lib = library.load()
+            part_o = torch.empty(int(lib.ra_attention_prefill_part_floats(num_heads, num_kv_heads, head_dim, n_slots, 0)),
+                                 dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(int(lib.ra_attention_prefill_part_floats(num_heads, num_kv_heads, head_dim, n_slots, 1)),
+                                  dtype=torch.float32, device=q.device)
+            library.call("ra_attention_prefill_split", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
+                         kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
+                         tiles.data_ptr(), int(n_tiles), ranges.data_ptr(), merge.data_ptr(), int(n_merge),
+                         part_o.data_ptr(), part_ml.data_ptr(), kcache.shape[2] * 16, num_heads, num_kv_heads,
+                         head_dim, float(scale), int(window), _stream())
+            return
         library.call("ra_attention_prefill", q.data_ptr(), q_stride, out.data_ptr(), out.stride(0),
                      kcache.data_ptr(), vcache.data_ptr(), tables.data_ptr(), tables.shape[1],
                      tiles.data_ptr(), int(n_tiles), kcache.shape[2] * 16, num_heads, num_kv_heads, head_dim,

@@ -320,6 +320,44 @@ def test_thousands_of_tokens_of_context(tmp_path, which, dtype):
     assert rel_err(got[-64:], ref[-64:]) < TOL[dtype]
 
 
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_short_portions_deep_in_a_long_prompt(tmp_path, which, monkeypatch):
+    """Portions of tens to hundreds of tokens behind thousands of cached ones, beside another request's
+    from its start: few query tiles with many keys each, which the prompt kernel takes cut by keys, a
+    second kernel adding the parts. The steps' plans are watched: tiles cut by keys must have occurred."""
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.weights import write_model_folder
+    dtype = "bfloat16"
+    raw = dict(TINY[which][0], max_position_embeddings=8192)
+    folder = str(tmp_path / "deep")
+    write_model_folder(config_from_dict(raw), 21, folder, dtype=dtype)
+    rawr, weights = read_folder(folder)
+    seqs = {"r": random_tokens(3400, raw["vocab_size"], 31), "s": random_tokens(900, raw["vocab_size"], 32)}
+    plan = [[("r", 2048)], [("r", 100), ("s", 300)], [("r", 40), ("s", 5)], [("r", 700), ("s", 200)],
+            [("s", 395), ("r", 70)], [("r", 442)]]
+    assert sum(n for st in plan for r, n in st if r == "r") == 3400 and sum(n for st in plan for r, n in st if r == "s") == 900
+    ops = kernels.current()
+    seen = {"cut": 0, "other": 0}
+    inner = ops.attention_prefill
+
+    def watched(q, q_stride, out, kc, vc, batch, Hq, Hkv, d, scale, window, group, tiles, n_tiles, ranges=None,
+                merge=None, n_merge=0, n_slots=0):
+        seen["cut" if n_slots else "other"] += 1
+        return inner(q, q_stride, out, kc, vc, batch, Hq, Hkv, d, scale, window, group, tiles, n_tiles, ranges,
+                     merge, n_merge, n_slots)
+    monkeypatch.setattr(ops, "attention_prefill", watched)
+    runner = ModelRunner.from_folder(folder, dtype=dtype, device="cuda:0", max_tokens=4352)
+    got = run_plan(runner, seqs, plan)
+    assert seen["cut"] > 0
+    for r, toks in seqs.items():
+        ref = plain.forward(rawr, weights, toks).float()
+        assert rel_err(got[r], ref) < TOL[dtype], r
+        for lo in (2048, 2148, 2188, 2888, 2958):           # the first token of each deep portion, and its last
+            if r == "r":
+                assert rel_err(got[r][lo:lo + 1], ref[lo:lo + 1]) < TOL[dtype]
+                assert rel_err(got[r][lo - 1:lo], ref[lo - 1:lo]) < TOL[dtype]
+
+
 @pytest.mark.parametrize("limit,n", [(300, 299), (100, 99)])
 def test_context_limit_that_is_no_power_of_two(folders, plain_cache, limit, n):
     """Captured decode steps pad the context to buckets (powers of two from 256); the last bucket is the

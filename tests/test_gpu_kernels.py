@@ -832,6 +832,30 @@ def test_attention_prefill(Hq, Hkv, d):
                                     tiles, len(info) // 4)
             ref = attention_reference(q, kc, vc, tables, q_lens, starts, Hq, Hkv, d, scale, window)
             close(out, ref, 2 ** -7)
+            # the same tiles cut by keys into parts of 1, 2 or 3 rounds of 64 (every other tile whole), listed in
+            # another order, their sums added by the second kernel
+            for per in (1, 2, 3):
+                items, ranges, merge, n_slots = [], [], [], 0
+                for k in range(len(info) // 4):
+                    i, row, n, pos = info[4 * k:4 * k + 4]
+                    r = -(-(pos + n) // 64)
+                    parts = -(-r // per)
+                    if k % 2 == 1 or parts < 2:
+                        items.append(((i, row, n, pos), (0, 1 << 30, -1)))
+                        continue
+                    merge += [row, n, n_slots, parts]
+                    for c in range(parts):
+                        items.append(((i, row, n, pos), (c * per * 64, (c + 1) * per * 64 if c + 1 < parts else 1 << 30, n_slots + c)))
+                    n_slots += parts
+                if not merge:
+                    continue
+                items = items[::-1]
+                out3 = torch.full((T, Hq * d), float("nan"), device=DEV, dtype=torch.bfloat16)
+                ops().attention_prefill(q.view(T, Hq * d), Hq * d, out3, kt(kc), vt(vc), batch, Hq, Hkv, d, scale, window, 0,
+                                        torch.tensor([v for it in items for v in it[0]], dtype=torch.int32, device=DEV), len(items),
+                                        torch.tensor([v for it in items for v in it[1]], dtype=torch.int32, device=DEV),
+                                        torch.tensor(merge, dtype=torch.int32, device=DEV), len(merge) // 4, n_slots)
+                close(out3, ref, 2 ** -7)
             if kernels.library.load().ra_attention_prefill_columns(Hq, Hkv, d) == 2 and window != 100:
                 # every other tile given to two workgroups, each with one of a wave's two column tiles
                 cut = []
