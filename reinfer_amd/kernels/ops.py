@@ -621,7 +621,8 @@ class HipKernels:
 
     def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False, row_sums=None,
                       emit=None, wide: Optional[bool] = None) -> None:
-        """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to.
+        """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to (with more rows
+        than the weight-streaming kernels take, by the library's product).
 
         An RMSNorm can ride on the products around it, y = rstd[m] * ((x .* w) . W^T):
         ``row_sums`` = (ss float32 [parts, M], eps, width) scales result row m by
@@ -634,6 +635,11 @@ class HipKernels:
             raise TypeError("linear_skinny: bfloat16 only")
         if accumulate and out.dtype != torch.float32:
             raise TypeError("linear_skinny: accumulation is into a float32 matrix")
+        if accumulate and M > 64 and bias is None and row_sums is None and emit is None and wide is None \
+                and not bool(library.load().ra_gemm_wide_preferred(2, M, N, K)):
+            # more rows than the weight-streaming kernels take: the library's product, adding in place
+            torch.addmm(out, x, weight.t(), out_dtype=torch.float32, out=out)
+            return None
         if row_sums is None and emit is None:
             self._few_rows("linear output", x, weight, bias, out, 2 if accumulate else 0, M, N, K, wide)
             return None
@@ -733,8 +739,16 @@ class HipKernels:
                 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1):
             return False
         M, K = x.shape
-        # above 64 rows only where the kernel that cuts K into ranges beats the library's product and an add
-        return M <= 64 or bool(library.load().ra_gemm_wide_preferred(2, M, weight.shape[0], K))
+        # above 64 rows where the kernel that cuts K into ranges beats the library's product and an add,
+        # or where the library's own product adds into the float matrix
+        return M <= 64 or M <= self.LIBRARY_ACCUMULATES_ROWS \
+            or bool(library.load().ra_gemm_wide_preferred(2, M, weight.shape[0], K))
+
+    # Rows up to which the library's product adds into the float residual stream itself (bfloat16 operands, a
+    # float matrix read and written): up to here it takes as long as the product with a bfloat16 result
+    # (2048 rows, 4096 x 4096: 67 against 69 us; 4096 x 12288: 187 against 191), and the norm kernel behind it
+    # reads one matrix less; at 8192 rows it is the slower one (218 against 179 us, 620 against 539).
+    LIBRARY_ACCUMULATES_ROWS = 4096
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 

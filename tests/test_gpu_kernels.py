@@ -675,8 +675,8 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
 @pytest.mark.parametrize("M", [65, 96, 97, 128])
 def test_accumulating_product_over_k_ranges_above_64_rows(M):
     """65 to 128 rows: a product that adds into the float stream over a long K is cut into K ranges (six or
-    eight row tiles) where that beats the library's product and an add; other products of that many rows
-    are not taken."""
+    eight row tiles) where that beats the library's product; other products of that many rows add into the
+    stream through the library's product."""
     lib = kernels.library.load()
     N, K = 2048, 12288
     assert lib.ra_gemm_wide_preferred(2, M, N, K) == 1
@@ -690,10 +690,31 @@ def test_accumulating_product_over_k_ranges_above_64_rows(M):
     assert ops().can_accumulate(x, w)
     ops().linear_skinny(x, w, stream, accumulate=True)
     close(stream, want, 2 ** -8)
-    small = torch.randn(512, 1024, device=DEV).to(torch.bfloat16)
-    assert not ops().can_accumulate(x[:, :1024], small)
-    with pytest.raises(kernels.KernelLibraryError, match="rows"):
-        ops().linear_skinny(x[:, :1024], small, torch.zeros(M, 512, device=DEV), accumulate=True)
+    small = (torch.randn(512, 1024, device=DEV) / 32).to(torch.bfloat16)
+    assert ops().can_accumulate(x[:, :1024], small)
+    stream = torch.randn(M, 512, device=DEV)
+    want = stream.double() + x[:, :1024].double() @ small.double().T
+    ops().linear_skinny(x[:, :1024], small, stream, accumulate=True)
+    close(stream, want, 2 ** -8)
+    with pytest.raises(kernels.KernelLibraryError, match="rows"):          # the kernel whose waves split K, asked by name
+        ops().linear_skinny(x[:, :1024], small, stream, accumulate=True, wide=False)
+    ops().linear_skinny(x[:, :1024], small, stream, accumulate=True, wide=True)      # and the other one
+    close(stream, want + x[:, :1024].double() @ small.double().T, 2 ** -8)
+
+
+@pytest.mark.parametrize("M,N,K", [(129, 520, 264), (700, 96, 1000), (2048, 1024, 4096), (4096, 80, 176)])
+def test_accumulating_product_of_many_rows_adds_in_the_library(M, N, K):
+    """More rows than the weight-streaming kernels take: the library's product reads and writes the float
+    stream itself (bfloat16 operands, float sums), so the addend is never rounded to bfloat16."""
+    torch.manual_seed(M + N)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    stream = torch.randn(M, N, device=DEV) * 100                # a bfloat16 addend beside 100 would show at 2**-8
+    want = stream.double() + x.double() @ w.double().T
+    assert ops().can_accumulate(x, w)
+    assert not ops().can_accumulate(torch.empty(ops().LIBRARY_ACCUMULATES_ROWS + 1, K, device=DEV, dtype=torch.bfloat16), w)
+    assert ops().linear_skinny(x, w, stream, accumulate=True) is None
+    assert (stream.double() - want).abs().max().item() < 2e-3
 
 
 @pytest.mark.parametrize("M", [3, 12, 40])
