@@ -120,6 +120,52 @@ def test_whole_model_special_cases(tmp_path):
     assert torch.equal(plain.forward(rawA, wA, toksA), plain.forward(untied, wA2, toksA))
 
 
+def one_layer(raw, w):
+    """The same model cut down to its first layer."""
+    raw1 = dict(raw, num_hidden_layers=1)
+    if "layer_types" in raw1:
+        raw1["layer_types"] = raw1["layer_types"][:1]
+    return raw1, {k: v for k, v in w.items() if not k.startswith("model.layers.") or k.startswith("model.layers.0.")}
+
+
+def test_one_layer_in_closed_form(tmp_path):
+    """Where the arrangement of a block shows in a formula that does not go through plain.forward's loop
+    (crates/cuda/src/engine.rs:4075-4314): pre-norm blocks that add into the stream."""
+    for which in ("A", "C"):
+        raw, w = read_folder(make_folder(tmp_path / which, which, "float32"))
+        raw1, w1 = one_layer(raw, w)
+        eps = raw["rms_norm_eps"]
+        dd = {k: v.double() for k, v in w1.items()}
+        L = "model.layers.0."
+        head = dd.get("lm_head.weight", dd["model.embed_tokens.weight"])
+        toks = random_tokens(10, raw["vocab_size"], 3)
+        x = dd["model.embed_tokens.weight"][torch.tensor(toks)]
+        # the attention's output projection zero: x + mlp(norm2(x)), the second norm taken of the stream itself
+        # (a norm of the block's output instead, or a feed-forward without the residual, gives something else)
+        w_no_attn = dict(w1)
+        w_no_attn[L + "self_attn.o_proj.weight"] = torch.zeros_like(w1[L + "self_attn.o_proj.weight"])
+        y = x + plain.swiglu(plain.rms_norm(x, dd[L + "post_attention_layernorm.weight"], eps),
+                             dd[L + "mlp.gate_proj.weight"], dd[L + "mlp.up_proj.weight"], dd[L + "mlp.down_proj.weight"])
+        want = plain.rms_norm(y, dd["model.norm.weight"], eps) @ head.T
+        assert torch.allclose(plain.forward(raw1, w_no_attn, toks), want, rtol=1e-9, atol=1e-9)
+        # one token, the down projection zero: the softmax over one key is 1, so query, key, their norms and the
+        # rotation drop out and head h returns the value of KV head h // (heads / KV heads), in head order
+        w_no_mlp = dict(w1)
+        w_no_mlp[L + "mlp.down_proj.weight"] = torch.zeros_like(w1[L + "mlp.down_proj.weight"])
+        H, KV, d = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
+        x0 = x[:1]
+        v = (plain.rms_norm(x0, dd[L + "input_layernorm.weight"], eps) @ dd[L + "self_attn.v_proj.weight"].T).view(KV, d)
+        heads = torch.stack([v[h // (H // KV)] for h in range(H)]).reshape(1, H * d)
+        y0 = x0 + heads @ dd[L + "self_attn.o_proj.weight"].T
+        want0 = plain.rms_norm(y0, dd["model.norm.weight"], eps) @ head.T
+        got0 = plain.forward(raw1, w_no_mlp, toks[:1], start_pos=5)
+        assert torch.allclose(got0, want0, rtol=1e-9, atol=1e-9)
+        # the other pairing of heads and KV heads (h % KV heads) is a different result for these weights
+        if KV > 1 and H // KV > 1:
+            wrong = torch.stack([v[h % KV] for h in range(H)]).reshape(1, H * d)
+            assert not torch.allclose(wrong, heads)
+
+
 def test_splitmix_vectors_and_greedy_ties():
     """crates/scheduler/src/rng.rs:83-87."""
     assert plain.splitmix64(0) == 0xE220A8397B1DCDAF
