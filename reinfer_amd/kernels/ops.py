@@ -741,13 +741,16 @@ class HipKernels:
         M, K = x.shape
         # above 64 rows where the kernel that cuts K into ranges beats the library's product and an add,
         # or where the library's own product adds into the float matrix
-        return M <= 64 or M <= self.LIBRARY_ACCUMULATES_ROWS \
+        return M <= 64 or self.LIBRARY_ACCUMULATES_FROM <= M <= self.LIBRARY_ACCUMULATES_ROWS \
             or bool(library.load().ra_gemm_wide_preferred(2, M, weight.shape[0], K))
 
     # Rows up to which the library's product adds into the float residual stream itself (bfloat16 operands, a
     # float matrix read and written): up to here it takes as long as the product with a bfloat16 result
     # (2048 rows, 4096 x 4096: 67 against 69 us; 4096 x 12288: 187 against 191), and the norm kernel behind it
     # reads one matrix less; at 8192 rows it is the slower one (218 against 179 us, 620 against 539).
+    # Below 129 rows (decode steps of 65 to 128 requests) it is a wash (a step of 96 requests 11.78 against
+    # 11.69 ms with the norm kernel's add, of 128 requests 14.28 against 14.36): those steps stay as they were.
+    LIBRARY_ACCUMULATES_FROM = 129
     LIBRARY_ACCUMULATES_ROWS = 4096
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear

@@ -675,8 +675,8 @@ def test_wide_gated_product_takes_the_many_partial_sums_of_a_narrow_producer(M):
 @pytest.mark.parametrize("M", [65, 96, 97, 128])
 def test_accumulating_product_over_k_ranges_above_64_rows(M):
     """65 to 128 rows: a product that adds into the float stream over a long K is cut into K ranges (six or
-    eight row tiles) where that beats the library's product; other products of that many rows add into the
-    stream through the library's product."""
+    eight row tiles) where that beats the library's product; other products of that many rows are not offered
+    (asked for all the same, they add into the stream through the library's product)."""
     lib = kernels.library.load()
     N, K = 2048, 12288
     assert lib.ra_gemm_wide_preferred(2, M, N, K) == 1
@@ -691,7 +691,7 @@ def test_accumulating_product_over_k_ranges_above_64_rows(M):
     ops().linear_skinny(x, w, stream, accumulate=True)
     close(stream, want, 2 ** -8)
     small = (torch.randn(512, 1024, device=DEV) / 32).to(torch.bfloat16)
-    assert ops().can_accumulate(x[:, :1024], small)
+    assert not ops().can_accumulate(x[:, :1024], small)         # the library's product and the norm kernel's add are faster
     stream = torch.randn(M, 512, device=DEV)
     want = stream.double() + x[:, :1024].double() @ small.double().T
     ops().linear_skinny(x[:, :1024], small, stream, accumulate=True)
