@@ -747,11 +747,12 @@ class HipKernels:
     # Rows up to which the library's product adds into the float residual stream itself (bfloat16 operands, a
     # float matrix read and written): up to here it takes as long as the product with a bfloat16 result
     # (2048 rows, 4096 x 4096: 67 against 69 us; 4096 x 12288: 187 against 191), and the norm kernel behind it
-    # reads one matrix less; at 8192 rows it is the slower one (218 against 179 us, 620 against 539).
+    # reads one matrix less (3072 rows: 95 against 85 and 248 against 275 us); from 4096 rows on it is the slower one
+    # (4096: 116 against 95 and 314 against 279 us; 8192: 218 against 179, 620 against 539).
     # Below 129 rows (decode steps of 65 to 128 requests) it is a wash (a step of 96 requests 11.78 against
     # 11.69 ms with the norm kernel's add, of 128 requests 14.28 against 14.36): those steps stay as they were.
     LIBRARY_ACCUMULATES_FROM = 129
-    LIBRARY_ACCUMULATES_ROWS = 4096
+    LIBRARY_ACCUMULATES_ROWS = 3072
 
     GATE_GROUP = 8        # rows of gate, then rows of up, in the weight of gated_linear
 
