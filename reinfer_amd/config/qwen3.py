@@ -78,6 +78,11 @@ class Qwen3Config:
         # what the engine has no part for must be off, not silently ignored
         if read_bool(cfg, "attention_bias", False):
             raise ConfigError("attention_bias", "Qwen3 projections carry no bias; true is not supported")
+        act = cfg.get("hidden_act", None)
+        if act is not None and act != "silu":
+            # the gate of the feed-forward is SiLU in every kernel (the reference fixes it the same way,
+            # crates/cuda/kernels/dense_kernels.cu:202-213, and never reads the key)
+            raise ConfigError("hidden_act", f"the feed-forward's gate is SiLU; {act!r} is not supported")
         scaling = cfg.get("rope_scaling", None)
         if scaling not in (None, {}):
             kind = scaling.get("rope_type", scaling.get("type")) if isinstance(scaling, dict) else scaling

@@ -67,6 +67,7 @@ def test_missing_key_names_the_key(key):
     ({"head_dim": 15}, "head_dim"), ({"hidden_size": "64"}, "hidden_size"),
     ({"use_sliding_window": True}, "sliding_window"), ({"layer_types": ["full_attention"]}, "layer_types"),
     ({"tie_word_embeddings": "yes"}, "tie_word_embeddings"),
+    ({"hidden_act": "gelu"}, "hidden_act"), ({"hidden_act": 3}, "hidden_act"),
 ])
 def test_bad_values_are_refused(patch, key):
     raw = dict(TINY_A)

@@ -248,3 +248,72 @@ def test_the_engine_hands_back_the_weights_it_was_built_from(tmp_path):
     for decl in (ParamDecl("m.weight", (5000, 4099)), ParamDecl("v.weight", (4097,), init="norm", role="vector")):
         for dt in (torch.float32, torch.bfloat16):
             assert torch.equal(random_tensor(decl, 3, dt, torch.device("cuda:0")).cpu(), random_tensor(decl, 3, dt)), decl.name
+
+
+@pytest.fixture(scope="module")
+def w8_long():
+    """One layer of the 8B widths with room for positions up to 8,700."""
+    SHAPES["8b_long"] = dict(raw_config(1, 4096, 32, 12288, False), max_position_embeddings=8704)
+    w = Width("8b_long", max_tokens=8704, max_seqs=4)
+    yield w
+    del w
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_of_thousands_of_tokens_at_the_8b_widths(w8_long, dtype):
+    """Steps longer than any other test feeds, at the rows where the dispatch changes: 8,192 tokens in one
+    step (what the bench's 8,192-token prompt point runs: the output and down projections no longer add into the
+    stream through the library, four times the query tiles the chip holds at once, the row kernels at 8,192 rows)
+    from position 0 and behind 300 cached tokens; 4,096; and 3,072 and 3,073 rows, the last step whose library
+    products add into the stream and the first whose do not, each from position 0 and behind earlier context.
+    Logits at the first and last row of every step and at a spread between, against the plain implementation."""
+    n = 8492
+    seqs = {"xl": w8_long.seq("xl", n, 41)}
+    plans = [[8192, 300], [300, 8192], [3072, 3073, 2347], [3073, 4096, 1323]]
+    edges = set()
+    for plan in plans:
+        at = 0
+        for k in plan:
+            edges |= {at, at + 1, at + k - 1}
+            at += k
+    wanted = {"xl": sorted(edges | {63, 64, 1000, 2047, 2048, 4095, 4500, 5555, 6143, 6144, 7000, 8000, 8191, n - 2})}
+    for plan in plans:
+        check(w8_long, dtype, seqs, [[("xl", k)] for k in plan], wanted)
+
+
+def test_decoding_requests_beside_two_prompt_portions_at_the_8b_widths(w8):
+    """The step a serving run makes all the time: ten (then eight) requests decode while two others bring
+    portions of their prompts, several steps in a row; with eight or more single tokens beside prompt tiles the
+    decode attention runs on a second stream beside the prompt attention. Two decoding requests end in the
+    middle and a new prompt starts on their blocks (the allocator hands the last freed out first); the keys and
+    values of every freed block are overwritten with NaN at once, so a read of a stale slot shows."""
+    for dtype in ("bfloat16", "float32"):
+        runner = w8.runners[dtype]
+        runner.poison_freed_blocks(True)
+        try:
+            dec = {f"d{i}": w8.seq(f"d{i}", 200 + 13 * i + 12, 60 + i) for i in range(10)}
+            pro = {"p1": w8.seq("p1", 700, 71), "p2": w8.seq("p2", 500, 72), "p3": w8.seq("p3", 450, 73)}
+            seqs = dict(dec, **pro)
+            tail = 12                                         # each decoding request's last 12 tokens come one by one
+            plan = [[(r, len(s) - tail) for r, s in list(dec.items())[lo:lo + 5]] for lo in (0, 5)]
+            ones = [(r, 1) for r in dec]
+            plan += [ones + [("p1", 256), ("p2", 200)], ones + [("p1", 256), ("p2", 200)],
+                     ones + [("p1", 187), ("p2", 99)], ones + [("p1", 1), ("p2", 1)]]
+            # d0 and d1 are cut short here: they end (in `ends`) and p3 starts on their blocks
+            ones8 = [(r, 1) for r in dec if r not in ("d0", "d1")]
+            plan += [ones8 + [("p3", 300)], ones8 + [("p3", 148)]] + [ones8 + [("p3", 1)]] * 2
+            plan += [ones8] * 4
+            wanted = {r: list(range(len(s) - tail, len(s))) for r, s in dec.items()}
+            wanted["d0"] = wanted["d0"][:4]
+            wanted["d1"] = wanted["d1"][:4]
+            wanted.update({"p1": [0, 255, 256, 511, 512, 698, 699], "p2": [0, 199, 200, 399, 400, 498, 499],
+                           "p3": [0, 1, 299, 300, 447, 448, 449]})
+            short = dict(seqs, d0=seqs["d0"][:len(seqs["d0"]) - tail + 4], d1=seqs["d1"][:len(seqs["d1"]) - tail + 4])
+            got = feed(runner, short, plan, wanted)
+            for r in seqs:
+                err = rel_err(got[r], w8.plain_rows(r, wanted[r]))
+                assert err < TOL[dtype], (r, dtype, err)
+            runner.manager.check()
+        finally:
+            runner.poison_freed_blocks(False)

@@ -283,6 +283,53 @@ def test_qk_norm_rope_cache_from_the_ranges_of_a_split_product(Hq, Hkv, d, rot, 
     assert int(torch.isnan(kc.float()).any(-1).sum()) == (nblk * bs - (T - 1)) * Hkv
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rotation_by_hand_through_the_position_part_and_the_cache_index(dtype):
+    """Numbers written out, not computed by the expression under test: head size 16, theta 10000, so pair j
+    turns by position * 10^(-j/2) (crates/kernels/src/refs.rs:25-37: the exponent is -2j over the whole head
+    size). Position 3: pair 6 turns by 0.003, pair 2 by 0.3. The frequencies come from the position part the
+    engine builds, and the key is read back from the cache by the index formula of csrc/common.h
+    (K tile [d/8][16 slots][8], V tile [d/16][4][16][4]) spelt out here, not through cache.layout."""
+    from reinfer_amd.config.schema import PositionSpec
+    from reinfer_amd.parts import lookup
+    d, bs, nblk = 16, 32, 3
+    part = lookup("position", "rope_neox")(PositionSpec("rope_neox", rotary_dim=d, theta=10000.0), torch.device(DEV))
+    assert torch.allclose(part.inv_freq.cpu().double(), torch.tensor(
+        [1.0, 0.31622776601683794, 0.1, 0.031622776601683794, 0.01, 0.0031622776601683794, 0.001,
+         0.00031622776601683794], dtype=torch.float64), rtol=1e-7, atol=0)
+    qkv = torch.zeros(1, 3 * d, device=DEV)
+    qkv[0, 6] = 1.0                     # q = e_6: a of pair 6
+    qkv[0, d + 10] = 2.0                # k = 2 e_10: b of pair 2
+    qkv[0, 2 * d:] = torch.arange(1, d + 1)
+    qkv = qkv.to(DT[dtype])
+    kc = torch.full((nblk, 1, bs // 16, 16 * d), float("nan"), device=DEV, dtype=DT[dtype])
+    vc = torch.full_like(kc, float("nan"))
+    block, off = 1, 21                  # the second tile of the block, slot 5 of the tile
+    ops().qk_norm_rope_cache(qkv, None, None, 0.0, torch.tensor([3], dtype=torch.int32, device=DEV), part.inv_freq,
+                             part.rotary_dim, part.style, torch.tensor([block * bs + off], dtype=torch.int32, device=DEV),
+                             kc, vc, 1, 1, d)
+    tol = 1e-6 if dtype == "float32" else 2 ** -8
+    q = qkv[0, :d].double().cpu()
+    want_q = torch.zeros(d, dtype=torch.float64)
+    want_q[6], want_q[14] = 0.999995500003375, 0.002999995500002025            # cos 0.003, sin 0.003
+    assert (q - want_q).abs().max().item() <= tol
+    want_k = torch.zeros(d, dtype=torch.float64)
+    want_k[2], want_k[10] = -2 * 0.29552020666133955, 2 * 0.955336489125606    # -b sin 0.3, b cos 0.3
+    kflat, vflat = kc[block, 0].reshape(-1).double().cpu(), vc[block, 0].reshape(-1).double().cpu()
+    seen_k, seen_v = set(), set()
+    for e in range(d):
+        ik = (off // 16) * 16 * d + ((e // 8) * 16 + off % 16) * 8 + e % 8
+        iv = (off // 16) * 16 * d + (((e // 16) * 4 + (off % 16) // 4) * 16 + e % 16) * 4 + (off % 16) % 4
+        assert abs(kflat[ik].item() - want_k[e].item()) <= tol, (e, kflat[ik].item(), want_k[e].item())
+        assert vflat[iv].item() == float(e + 1)
+        seen_k.add(ik)
+        seen_v.add(iv)
+    assert len(seen_k) == d and len(seen_v) == d
+    # nothing else of the cache was written
+    assert int((~torch.isnan(kflat)).sum()) == d and int((~torch.isnan(vflat)).sum()) == d
+    assert torch.isnan(kc[[0, 2]].float()).all() and torch.isnan(vc[[0, 2]].float()).all()
+
+
 def test_rotation_depends_on_distance_only():
     """<R_p q, R_t k> is a function of p - t: shift all positions and nothing changes."""
     Hq, Hkv, d, bs = 2, 1, 32, 16

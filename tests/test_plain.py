@@ -187,3 +187,77 @@ def test_logit_bias_is_added_first_and_validated():
     with pytest.raises(ValueError, match="twice"):
         SamplingParams(logit_bias=((1, 0.5), (1, 0.25)))
     assert not SamplingParams().filters
+
+
+def test_rope_frequency_schedule_by_hand():
+    """The frequency of pair j is theta^(-2j/d) with d the whole head size (crates/kernels/src/refs.rs:25-37:
+    ``exp = -(2 p) / (2 half)``; crates/cuda/tests/engine_vs_cpu.rs:291-299). The numbers below are written out,
+    not computed from the same expression: theta^(-j/d), or d/2 in the denominator, gives others."""
+    # d = 4, theta = 10000, position 1: frequencies [1, 0.01]
+    e = torch.eye(4, dtype=D).view(4, 1, 4)
+    y = plain.rope_neox(e, torch.tensor([1, 1, 1, 1]), 10000.0)[:, 0]
+    cos1, sin1 = 0.5403023058681398, 0.8414709848078965
+    cos001, sin001 = 0.9999500004166653, 0.009999833334166664
+    want = torch.tensor([[cos1, 0.0, sin1, 0.0],          # unit vector 0: a = 1, b = 0 of pair 0
+                         [0.0, cos001, 0.0, sin001],      # unit vector 1: pair 1 turns by 0.01, not by 1 or 0.1
+                         [-sin1, 0.0, cos1, 0.0],         # unit vector 2 = b of pair 0: out[0] = -b sin
+                         [0.0, -sin001, 0.0, cos001]], dtype=D)
+    assert torch.allclose(y, want, rtol=0, atol=1e-15)
+    # d = 8, theta = 10000, position 3, pair 3: frequency 10000^(-6/8) = 0.001, angle 0.003
+    u = torch.zeros(1, 1, 8, dtype=D)
+    u[0, 0, 3] = 1.0
+    y = plain.rope_neox(u, torch.tensor([3]), 10000.0)[0, 0]
+    assert abs(y[3].item() - 0.999995500003375) < 1e-15 and abs(y[7].item() - 0.002999995500002025) < 1e-15
+    assert y[[0, 1, 2, 4, 5, 6]].abs().max().item() == 0.0
+    # pair 1 of the same: 10000^(-2/8) = 0.1, angle 0.3
+    u = torch.zeros(1, 1, 8, dtype=D)
+    u[0, 0, 5] = 2.0
+    y = plain.rope_neox(u, torch.tensor([3]), 10000.0)[0, 0]
+    assert abs(y[1].item() + 2 * 0.29552020666133955) < 1e-15 and abs(y[5].item() - 2 * 0.955336489125606) < 1e-15
+
+
+def _two_token_block(d_scale_q: float = 1.0):
+    """One head of size 4, all projections the identity (q's scaled by ``d_scale_q``), norm weights 1."""
+    eye = torch.eye(4, dtype=D)
+    return {"L.self_attn.q_proj.weight": eye * d_scale_q, "L.self_attn.k_proj.weight": eye,
+            "L.self_attn.v_proj.weight": eye, "L.self_attn.o_proj.weight": eye,
+            "L.self_attn.q_norm.weight": torch.ones(4, dtype=D), "L.self_attn.k_norm.weight": torch.ones(4, dtype=D)}
+
+
+def test_attention_scale_by_hand():
+    """Two keys, weights softmax([a, b] / sqrt(d)) written out (crates/cuda/tests/engine_vs_cpu.rs:203,
+    ``scale = 1 / sqrt(d)``, on the score before the softmax). Token 0 = [2,0,0,0] at position 0, token 1 =
+    [0,0,2,0] at position 1 (theta 10000, d = 4: pair 0 turns by 1 radian). Head norm with eps 0 leaves both
+    (mean square 1). q1 = k1 = [-2 sin 1, 0, 2 cos 1, 0], k0 = [2,0,0,0]: scores [-4 sin 1, 4], over sqrt(4):
+    [-1.682941969615793, 2]; the weight of key 1 is 1 / (1 + exp(-3.682941969615793)) = 0.9754680718274085.
+    Without the scale it would be 0.99937; with 1/d, 0.863."""
+    xn = torch.tensor([[2.0, 0, 0, 0], [0, 0, 2.0, 0]], dtype=D)
+    out = plain.attention_block(xn, torch.tensor([0, 1]), _two_token_block(), "L.", 1, 1, 4, 10000.0, 0.0, 0)
+    p1 = 0.9754680718274085
+    assert torch.allclose(out[0], xn[0], rtol=0, atol=1e-15)                 # one key: its value
+    want = (1 - p1) * xn[0] + p1 * xn[1]                                     # values are not rotated
+    assert torch.allclose(out[1], want, rtol=0, atol=1e-14), (out[1], want)
+
+
+def test_head_norm_eps_is_the_layer_eps_by_hand():
+    """The head norm's eps is rms_norm_eps, inside the root (crates/cuda/tests/engine_vs_cpu.rs:185-195 pass
+    ``cfg.rms_eps``). Queries of order 1e-3 (q's projection scaled by 1e-3) make it count: q = [2e-3, 0, 0, 0]
+    has mean square 1e-6, so with eps 1e-5 the normed q is 2e-3 / sqrt(1.1e-5) = 0.6030226891555273 (with
+    eps 0, or 1e-6, it would be 2 or 1.414). Both tokens [2,0,0,0]; keys 2 / sqrt(1 + 1e-5) = 1.9999900000749994.
+    Position 1 turns pair 0 by 1 radian: q1.k0 = |q||k| cos 1, q1.k1 = |q||k|; over sqrt(4) the scores differ
+    by |q||k| (1 - cos 1) / 2 = 0.27720...; the weight of key 1 is 1 / (1 + exp(-that))."""
+    w = _two_token_block(1e-3)
+    # Both tokens are [2,0,0,0]; the values must still tell the keys apart: a 1e-30 in token 1's last entry
+    # leaves norms and scores alone and is made 1 by the value projection. Values: token 0 [1,0,0,0], token 1 [1,1,0,0].
+    xn2 = torch.tensor([[2.0, 0, 0, 0], [2.0, 0, 0, 1e-30]], dtype=D)
+    vproj = torch.zeros(4, 4, dtype=D)
+    vproj[0, 0] = 0.5
+    vproj[1, 3] = 1e30
+    w["L.self_attn.v_proj.weight"] = vproj
+    out = plain.attention_block(xn2, torch.tensor([0, 1]), w, "L.", 1, 1, 4, 10000.0, 1e-5, 0)
+    q_len, k_len = 0.6030226891555273, 1.9999900000749994
+    gap = q_len * k_len * (1 - 0.5403023058681398) / 2.0
+    p1 = 1.0 / (1.0 + math.exp(-gap))
+    assert abs(out[1, 0].item() - 1.0) < 1e-12
+    assert abs(out[1, 1].item() - p1) < 1e-9, (out[1, 1].item(), p1)
+    assert abs(p1 - 0.5688) < 1e-3          # eps 0 would give 0.7149, eps 1e-6 0.6570

@@ -156,3 +156,45 @@ def test_trace_run_dumps_the_hidden_state_behind_every_layer(tmp_path, dtype):
         assert rel_err(got1[layer], want1[layer]) < TOL[dtype], layer
     # the logits files are what they are without the option
     assert (out / "1.f32").exists() and not (out / "0.f32").exists()
+
+
+def test_trace_run_checks_start_against_what_the_cache_holds(tmp_path):
+    """An entry may say where it starts. A right ``start`` changes nothing; a trace that skips tokens (or
+    repeats them, or starts a fresh request elsewhere than at 0) ends the replay with status 4 before that
+    step runs: the steps before it are answered, the bad one is not and leaves no file."""
+    folder = make_folder(tmp_path, "A", "float32")
+    raw, weights = read_folder(folder)
+    V = raw["vocab_size"]
+    a, b = random_tokens(20, V, 8), random_tokens(9, V, 9)
+    ref = plain.forward(raw, weights, a).float()
+
+    def run(steps, name):
+        out = tmp_path / name
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+             "--out", str(out), "--max-tokens", "128"],
+            input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+        return proc, out
+
+    good = [
+        {"step": 0, "entries": [{"id": "a", "start": 0, "tokens": a[:12], "want": [11]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "start": 12, "tokens": a[12:20], "want": [7]},
+                                {"id": "b", "tokens": b, "want": []}], "end": ["a"]},
+        # the id again after its end: a fresh request, which starts at 0
+        {"step": 2, "entries": [{"id": "a", "start": 0, "tokens": a[:3], "want": [2]},
+                                {"id": "b", "start": 9, "tokens": [1], "want": []}], "end": []},
+    ]
+    proc, out = run(good, "good")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = torch.from_numpy(np.fromfile(out / "1.f32", dtype="<f4").reshape(1, V))
+    assert rel_err(got, ref[19:20]) < TOL["float32"]
+
+    for name, bad in (("skips", {"id": "a", "start": 14, "tokens": a[14:20], "want": [5]}),
+                      ("repeats", {"id": "a", "start": 10, "tokens": a[10:20], "want": [9]}),
+                      ("fresh", {"id": "z", "start": 5, "tokens": a[5:9], "want": [3]})):
+        steps = [good[0], {"step": 1, "entries": [{"id": "b", "tokens": b, "want": [0]}, bad], "end": []}]
+        proc, out = run(steps, name)
+        assert proc.returncode == 4, (name, proc.returncode, proc.stderr[-2000:])
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0"]
+        assert (out / "0.f32").exists() and not (out / "1.f32").exists()
+        assert "start" in proc.stderr and repr(bad["id"]) in proc.stderr
