@@ -138,17 +138,26 @@ class FeedForwardSpec:
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """One layer: how norm, mixer and feed-forward are arranged, and its parts."""
+    """One layer: how norm, mixer and feed-forward are arranged, and its parts.
+
+    The four part records are what the "prenorm" arrangement is built from; another arrangement may
+    leave any of them out (one norm for both parts, a layer that only mixes) and bring a typed record
+    of its own in ``params`` (any frozen dataclass), or loose options in ``extra``."""
     kind: str                       # e.g. "prenorm": x += mixer(norm(x)); x += ffn(norm(x))
-    mixer: MixerSpec
-    ffn: FeedForwardSpec
-    mixer_norm: NormSpec
-    ffn_norm: NormSpec
-    prefix: str                     # tensor-name prefix of this block's weights
+    mixer: Optional[MixerSpec] = None
+    ffn: Optional[FeedForwardSpec] = None
+    mixer_norm: Optional[NormSpec] = None
+    ffn_norm: Optional[NormSpec] = None
+    prefix: str = ""                # tensor-name prefix of this block's weights
     mixer_prefix: str = "self_attn."
     ffn_prefix: str = "mlp."
     mixer_norm_name: str = "input_layernorm.weight"
     ffn_norm_name: str = "post_attention_layernorm.weight"
+    params: Any = None
+    extra: Tuple[Tuple[str, Any], ...] = ()
+
+    def option(self, name: str, default: Any = None) -> Any:
+        return dict(self.extra).get(name, default)
 
 
 @dataclass(frozen=True)

@@ -396,6 +396,9 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     lt += __shfl_xor(lt, 16, RA_WAVE);
     lt += __shfl_xor(lt, 32, RA_WAVE);
     if (slot >= 0) {
+      // (a workgroup that was given some of a wave's column tiles only leaves the others' columns alone: two
+      // workgroups with the halves of one part then fill one slot between them)
+      if (!((col_mask >> j) & 1)) continue;
       // a part: the sums as they are, for the kernel that adds the parts (a column without a query, or one
       // that saw none of this part's keys, leaves zeros and -inf or 0 as its maximum: both weigh nothing)
       const size_t col = ((size_t)slot * gy + by) * (FP_WAVES * NC * 16) + (wave * NC + j) * 16 + r;

@@ -72,6 +72,9 @@ __host__ __device__ __forceinline__ size_t cache_v_index(int off, int e, int d) 
 extern thread_local char ra_error_text[512];
 int ra_fail(const char* fmt, ...);
 
+// Compute units of the current device (cached per device; 256 if the device cannot be asked).
+int ra_cu_count(void);
+
 #define RA_CHECK(cond, ...)                    \
   do {                                         \
     if (!(cond)) return ra_fail(__VA_ARGS__);  \

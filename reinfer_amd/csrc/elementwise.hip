@@ -16,6 +16,18 @@ int ra_fail(const char* fmt, ...) {
 }
 
 extern "C" const char* ra_last_error(void) { return ra_error_text; }
+
+int ra_cu_count(void) {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
 extern "C" int ra_abi_version(void) { return RA_ABI_VERSION; }
 
 // ---------------------------------------------------------------------------

@@ -74,6 +74,10 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], const floa
   const int wave = threadIdx.x / RA_WAVE;
   const int r = lane & 15, g = lane >> 4;
   if (nf.in_ss) {
+    // In the persistent kernel this runs once a tile, and a wave may write row_ss for the next tile while
+    // wave 0 still reads it for this one, with no barrier between: that is safe because what is written
+    // does not depend on the tile (the sums of squares of the input rows are the same for every feature
+    // tile), so the racing write stores the value that is already there.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = mt * 16 + r;
@@ -586,17 +590,7 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
   return 0;
 }
 
-static int skinny_cus() {
-  static int cus[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cus[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus[dev] = n;
-  }
-  return cus[dev];
-}
+static int skinny_cus() { return ra_cu_count(); }
 
 template <int NT, int WAVES, int U, int DEPTH, int OCC, int MROWS>
 static int launch_deep(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int out_dtype,

@@ -322,16 +322,17 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
 // How [M, N, K] is cut: waves a workgroup (5 to 8, 16 features each) and K ranges. With many features
 // one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
 // workgroups of 96; 19456: 244 of 80; 51200: 458 of 112). With few features 128 a workgroup and the smallest power of two up to 8 of K
-// ranges that gives at least 192 workgroups, each range a multiple of the run and two runs or more.
+// ranges that gives at least three quarters as many workgroups as the chip has CUs (192 of 256), each range a multiple of the run and two runs or more.
 static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int* k_per_split, bool* partial = nullptr,
                      bool emits = false) {
   if (partial) *partial = emits;                       // the adding kernel writes what the next norm needs
+  const int cus = ra_cu_count(), fill = cus - cus / 4;  // workgroups that keep the chip busy: three quarters of its CUs
   const int cb8 = (N + 127) / 128;
   *waves = 8;
   *S = 1;
   *k_per_split = (K + GW_KS - 1) / GW_KS * GW_KS;
-  if ((cb8 >= 192 && !emits) || epilogue == WEPI_SILU_PAIRS) {
-    // The width whose workgroups fill whole rounds of the chip's 256 CUs best: 5 to 8 waves from 17 rows
+  if ((cb8 >= fill && !emits) || epilogue == WEPI_SILU_PAIRS) {
+    // The width whose workgroups fill whole rounds of the chip's CUs (256 on MI355X) best: 5 to 8 waves from 17 rows
     // on, 6 or 8 below (there the odd widths were slower inside a decode step although faster alone, and
     // a shape that neither 6 nor 8 fills well goes to gemm_skinny: ra_gemm_wide_preferred). A narrower
     // workgroup stages the activations more often, so it must fill the rounds clearly better (with many
@@ -342,7 +343,7 @@ static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int*
     for (int wv = 8; wv >= 5; --wv) {
       if (M <= 16 && (wv == 7 || wv == 5)) continue;
       const int cb = (N + wv * 16 - 1) / (wv * 16);
-      const double e = (double)cb / (((cb + 255) / 256) * 256);
+      const double e = (double)cb / (((cb + cus - 1) / cus) * cus);
       if (e > best * 1.03) {
         best = e;
         *waves = wv;
@@ -351,7 +352,7 @@ static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int*
     return;
   }
   int s = 1;
-  while (s < 8 && cb8 * s < 192 && K / (s * 2) >= 2 * GW_KS) s *= 2;
+  while (s < 8 && cb8 * s < fill && K / (s * 2) >= 2 * GW_KS) s *= 2;
   int kps = (K + s - 1) / s;
   kps = (kps + GW_KS - 1) / GW_KS * GW_KS;
   *S = (K + kps - 1) / kps;
@@ -366,10 +367,14 @@ extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
   if (M < 1 || M > 128) return 0;
   int waves, S, kps;
   gw_split(epilogue, M, N, K, &waves, &S, &kps);
+  // sizes are priced a CU: a product is "large" where every CU has more than 128 KiB of weights to stream
+  // (on 256 CUs: more than 4096 x 4096 bfloat16)
+  const int cus = ra_cu_count(), fill = cus - cus / 4;
+  const bool large = (long)N * K * 2 > 131072L * cus;
   // 65 to 128 rows: the library's products are as fast or faster (151936 x 4096 at 128 rows: 285 us against
   // 400) but for a product that adds into the residual stream over a long K, which this kernel cuts into
   // ranges (4096 x 12288 at 96 / 128 rows: 37 / 43 us against 59 / 70 for the library's product and the add)
-  if (M > 64) return (epilogue == WEPI_ACCUM && S > 1 && (long)N * K > 4096L * 4096L) ? 1 : 0;
+  if (M > 64) return (epilogue == WEPI_ACCUM && S > 1 && large) ? 1 : 0;
   // from 9 to 16 rows the gated product of a wide feed-forward (up to 8 rows the other kernel, whose
   // workgroups stay and keep two runs a wave in flight, is ahead: 24576 x 4096 36 us against 37, 51200 x
   // 5120 91 to 97 against 101 to 103): one K range, enough workgroups to fill the
@@ -379,10 +384,11 @@ extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
   // K = 2560 / 4096 / 5120: 148 / 237 / 280 us against 170 / 239 / 327)
   const int cb = (N + waves * 16 - 1) / (waves * 16);
   if (M < 17) {
-    if (epilogue == WEPI_SILU_PAIRS) return (M > 8 && S == 1 && cb >= 192 && cb * 10 >= ((cb + 255) / 256) * 256 * 8) ? 1 : 0;
-    return (epilogue == WEPI_PLAIN && M > 8 && S == 1 && cb >= 768) ? 1 : 0;
+    if (epilogue == WEPI_SILU_PAIRS)
+      return (M > 8 && S == 1 && cb >= fill && cb * 10 >= ((cb + cus - 1) / cus) * cus * 8) ? 1 : 0;
+    return (epilogue == WEPI_PLAIN && M > 8 && S == 1 && cb >= 3 * cus) ? 1 : 0;
   }
-  return (S == 1 || (long)N * K > 4096L * 4096L) ? 1 : 0;
+  return (S == 1 || large) ? 1 : 0;
 }
 
 // Floats of scratch that ra_gemm_wide needs for this product (0: none).

@@ -138,7 +138,11 @@ int ra_sample(const float* logits, int n_rows, int vocab, int row_stride, const 
 // hipFree or allocating routine; n_rows * ra_sample_slices(vocab) may be at most
 // ra_sample_static_max_pairs() (65536), more is refused with a message. All calls on one GPU share that
 // GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+// ra_sample_static_prepare() looks the array's address up for the current device (once per device, under
+// a lock); ra_sample_static does the same at its first call on a device, so a caller that captures its
+// stream calls prepare beforehand, outside the capture.
 long ra_sample_static_max_pairs(void);
+int ra_sample_static_prepare(void);
 int ra_sample_static(const float* logits, int n_rows, int vocab, int row_stride, const float* temperature,
                      const long long* seeds, const int* positions, int* tokens, hipStream_t stream);
 

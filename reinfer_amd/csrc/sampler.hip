@@ -162,6 +162,14 @@ static int static_scratch(void** out) {
 
 extern "C" long ra_sample_static_max_pairs(void) { return SAMPLE_STATIC_PAIRS; }
 
+// Looks the array's address up for the current device, so that no later call has to: a caller that will
+// run ra_sample_static under stream capture calls this once per device beforehand (a first call inside a
+// capture would make the lookup inside it).
+extern "C" int ra_sample_static_prepare(void) {
+  void* base = nullptr;
+  return static_scratch(&base);
+}
+
 extern "C" int ra_sample_static(const float* logits, int n_rows, int vocab, int row_stride,
                                 const float* temperature, const long long* seeds, const int* positions,
                                 int* tokens, hipStream_t stream) {

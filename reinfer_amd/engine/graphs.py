@@ -107,10 +107,8 @@ class _CapturedStep:
             block_tables=[dv(f"table{g}").view(B, W) for g in range(n_groups)],
             slots=[dv(f"slots{g}") for g in range(n_groups)],
             q_lens=[1] * B, starts=[ctx_cap - 1] * B, max_q_len=1, max_ctx_len=ctx_cap)
-        # the kernels choose grids from host-side numbers: fixed for this bucket
-        self.batch.extra["attention_plan"] = {
-            "n_decode": B, "decode_max_ctx": ctx_cap, "decode_list": None, "n_prefill": 0,
-            "prefill_list": None, "n_tiles": 0, "tiles": None}
+        # the kernels choose grids from host-side numbers: the parts fix them for this bucket
+        runner.model.plan_captured_step(self.batch, B, ctx_cap)
         self.logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.copied: Optional[torch.cuda.Event] = None      # behind the last copy out of the staging buffer

@@ -13,11 +13,10 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import torch
 
 from ..cache import CacheManager, OutOfBlocks, plan_groups
-from ..cache.layout import cache_shape
 from ..config import load_config
 from ..config.schema import ModelSpec
 from ..models import DecoderModel, declare_params
-from ..parts import KVNeed, LayerCache, StateNeed
+from ..parts import KVNeed, LayerCache, PagedNeed, StateNeed
 from ..weights import check_tensors, load_weights, random_tensor, random_tensors, storage_dtype, weight_from_folder
 from .._hostlib import StepError
 from .batch import StepBatch, StepEntry, build_step_batch
@@ -48,6 +47,7 @@ class ModelRunner:
         self.dtype = dtype
         self.device = device
         self._poison = False
+        self.last_logits: Optional[torch.Tensor] = None
         self._weight_source = ("given", weights)       # replaced by from_folder / from_config; see get_weight
         self.load_report: Dict[str, object] = {}
         self.block_size = int(block_size)
@@ -59,7 +59,7 @@ class ModelRunner:
         # which run-order entries keep keys of their own, and with which window
         windows: List[Optional[int]] = []
         for e, need in zip(spec.run_order, needs):
-            if isinstance(need, KVNeed) and e.cache_from is None:
+            if isinstance(need, (KVNeed, PagedNeed)) and e.cache_from is None:
                 windows.append(need.window)
             else:
                 windows.append(None)
@@ -77,24 +77,25 @@ class ModelRunner:
         self.num_blocks = int(num_blocks)
         self.manager = CacheManager(groups, self.block_size, [self.num_blocks] * len(groups), max_seqs)
 
-        # device side of the cache
+        # device side of the cache: what each mixer's need names, a tensor of [blocks, *one block] each
         self.caches: List[Optional[LayerCache]] = []
         for i, (e, need) in enumerate(zip(spec.run_order, needs)):
-            if isinstance(need, KVNeed):
+            if isinstance(need, (KVNeed, PagedNeed)):
                 if e.cache_from is None:
-                    # tiles of 16 slots in matrix-core operand order (cache/layout.py)
-                    shape = cache_shape(self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
-                    k = torch.zeros(shape, dtype=dtype, device=device)
-                    v = torch.zeros(shape, dtype=dtype, device=device)
-                    self.caches.append(LayerCache(k=k, v=v, group=group_of[i], writes=True))
+                    tensors = {}
+                    for name, shape, tdtype in need.block_tensors(self.block_size):
+                        tensors[name] = torch.zeros((self.num_blocks, *shape), dtype=tdtype or dtype, device=device)
+                    self.caches.append(LayerCache(k=tensors.get("k"), v=tensors.get("v"), group=group_of[i],
+                                                  writes=True, tensors=tensors))
                 else:
                     src = self.caches[e.cache_from]
                     src_need = needs[e.cache_from]
-                    if not isinstance(src_need, KVNeed) or (src_need.num_kv_heads, src_need.head_dim) != \
-                            (need.num_kv_heads, need.head_dim):
+                    if not isinstance(src_need, (KVNeed, PagedNeed)) or \
+                            tuple(src_need.block_tensors(self.block_size)) != tuple(need.block_tensors(self.block_size)):
                         raise ValueError(f"run entry {i} cannot read the cache of entry {e.cache_from}: "
                                          "different heads")
-                    self.caches.append(LayerCache(k=src.k, v=src.v, group=src.group, writes=False))
+                    self.caches.append(LayerCache(k=src.k, v=src.v, group=src.group, writes=False,
+                                                  tensors=src.tensors))
             elif isinstance(need, StateNeed):
                 state = torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device)
                 self.caches.append(LayerCache(state=state))
@@ -179,10 +180,10 @@ class ModelRunner:
         capacity = utilisation * total - weights, pages = capacity / page bytes
         (crates/memory/src/budget.rs:99-117)."""
         per_block = 0
-        size = torch.empty((), dtype=self.dtype).element_size()
         for need, w in zip(needs, windows):
             if w is not None:
-                per_block += 2 * need.num_kv_heads * self.block_size * need.head_dim * size
+                for _, shape, tdtype in need.block_tensors(self.block_size):
+                    per_block += math.prod(shape) * torch.empty((), dtype=tdtype or self.dtype).element_size()
         if per_block == 0:
             return 1
         if self.device.type != "cuda":
@@ -216,9 +217,10 @@ class ModelRunner:
                 continue
             idx = torch.tensor(sorted(set(blocks)), dtype=torch.long, device=self.device)
             for cache in self.caches:
-                if cache is not None and cache.k is not None and cache.writes and cache.group == g:
-                    cache.k[idx] = float("nan")
-                    cache.v[idx] = float("nan")
+                if cache is not None and cache.tensors and cache.writes and cache.group == g:
+                    for t in cache.tensors.values():
+                        if t.is_floating_point():
+                            t[idx] = float("nan")
 
     def has_request(self, rid: Hashable) -> bool:
         return rid in self.manager
@@ -263,6 +265,7 @@ class ModelRunner:
         self.manager.end_step(entries)
         if self._poison:
             self._poison_freed()           # blocks a window has passed
+        self.last_logits = logits          # for a caller that checks a run's results after timing it
         return logits, tokens
 
     def forward(self, batch: StepBatch, observer=None) -> torch.Tensor:

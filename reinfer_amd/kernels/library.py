@@ -84,6 +84,8 @@ def load() -> ctypes.CDLL:
         lib.ra_attention_prefill_part_floats.argtypes = [c_int, c_int, c_int, c_int, c_int]
         lib.ra_sample_static_max_pairs.restype = c_long
         lib.ra_sample_static_max_pairs.argtypes = []
+        lib.ra_sample_static_prepare.restype = c_int
+        lib.ra_sample_static_prepare.argtypes = []
         lib.ra_gemm_skinny_max_rows.restype = c_int
         lib.ra_gemm_skinny_max_rows.argtypes = []
         lib.ra_gemm_skinny_row_parts.restype = c_int

@@ -375,6 +375,13 @@ class HipKernels:
                     best, best_span = (items, merge, n_slots), span
         return best
 
+    def plan_captured_step(self, batch, num_rows: int, ctx_cap: int) -> None:
+        """The attention plan of a captured decode step: ``num_rows`` single tokens over contexts of at most
+        ``ctx_cap``, whatever the step that is replayed holds (the grids are chosen from these)."""
+        batch.extra["attention_plan"] = {
+            "n_decode": num_rows, "decode_max_ctx": ctx_cap, "decode_list": None, "n_prefill": 0,
+            "prefill_list": None, "n_tiles": 0, "tiles": None}
+
     def _attention_plan(self, batch, device, tile: int, room: int = 0, halves: bool = False):
         """Which tokens go to which kernel; made once per step and query-tile size, shared by the
         layers. ``room`` is the number of query tiles whose workgroups fill the chip once (0: the tiles

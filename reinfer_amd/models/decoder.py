@@ -59,13 +59,43 @@ class DecoderModel:
         self.run_order = spec.run_order
 
     def cache_needs(self) -> List[Optional[object]]:
-        """What each run-order entry keeps: KVNeed, StateNeed, or None."""
+        """What each run-order entry keeps: KVNeed, PagedNeed, StateNeed, or None. The block arrangement
+        answers (``cache_need()``); one that does not is asked for a ``mixer`` attribute's answer."""
         needs: List[Optional[object]] = []
         for e in self.run_order:
-            mixer = self.blocks[e.block].mixer
-            need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
-            needs.append(need)
+            block = self.blocks[e.block]
+            if hasattr(block, "cache_need"):
+                needs.append(block.cache_need())
+                continue
+            mixer = getattr(block, "mixer", None)
+            needs.append(mixer.cache_need() if mixer is not None and hasattr(mixer, "cache_need") else None)
         return needs
+
+    def parts(self):
+        """Every part of the model once: blocks, what they say they are made of, the norms and position part
+        at either end."""
+        seen, out = set(), []
+        def add(p):
+            if p is not None and id(p) not in seen:
+                seen.add(id(p))
+                out.append(p)
+        add(self.input_position)
+        for b in self.blocks:
+            add(b)
+            for p in (b.parts() if hasattr(b, "parts") else (getattr(b, "mixer", None), getattr(b, "ffn", None))):
+                add(p)
+        add(self.final_norm)
+        return out
+
+    def plan_captured_step(self, batch, num_rows: int, ctx_cap: int) -> None:
+        """A decode step that is captured once and replayed takes no host-side number from the step it
+        replays for: whatever a part's kernels choose grids or buffers by on the host must be fixed for the
+        bucket. Every part with a ``plan_captured_step(batch, num_rows, ctx_cap)`` is asked to write what it
+        needs into ``batch.extra`` (``num_rows`` requests of one token each, contexts of at most ``ctx_cap``)."""
+        for p in self.parts():
+            hook = getattr(p, "plan_captured_step", None)
+            if hook is not None:
+                hook(batch, num_rows, ctx_cap)
 
     def forward_layers(self, batch, caches: Sequence[Optional[LayerCache]], observer=None):
         """Embedding and all blocks: (residual stream, last addend not yet added).

@@ -73,6 +73,12 @@ class GroupedQueryAttention:
     def cache_need(self) -> KVNeed:
         return KVNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    def plan_captured_step(self, batch, num_rows: int, ctx_cap: int) -> None:
+        # the attention kernels pick their grids by host-side numbers of the step: the kernel set fixes them
+        hook = getattr(kernels.current(), "plan_captured_step", None)
+        if hook is not None:
+            hook(batch, num_rows, ctx_cap)
+
     def forward(self, x, batch, cache: LayerCache, resid: Optional[torch.Tensor] = None,
                 emit: Optional[NormTarget] = None):
         ops = kernels.current()

@@ -8,11 +8,35 @@ import torch
 
 
 @dataclass(frozen=True)
+class PagedNeed:
+    """Memory per token, in pages: the mixer names the tensors it keeps and the shape of one block of
+    each. ``tensors`` is a tuple of (name, shape of one block, dtype or None for the model's dtype), a -1
+    in a shape standing for the engine's block size; the
+    engine allocates ``[blocks, *shape]`` for each and hands them over in ``LayerCache.tensors`` by name;
+    token slot s of the step (``batch.slots[group]``) is slot ``s % block_size`` of block ``s // block_size``,
+    wherever in its block's shape the mixer puts it. ``window`` W > 0: only the last W tokens are read, the
+    blocks behind them go back to the pool."""
+    tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[torch.dtype]], ...]
+    window: int = 0
+
+    def block_tensors(self, block_size: int):
+        return tuple((name, tuple(block_size if n == -1 else n for n in shape), dtype)
+                     for name, shape, dtype in self.tensors)
+
+
+@dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of every token (``window`` 0) or of the last ``window`` tokens."""
+    """Keys and values of every token (``window`` 0) or of the last ``window`` tokens, as the attention
+    kernels read them: tensors "k" and "v", a block of each ``[kv_heads, block_size // 16, 16 * head_dim]``,
+    tiles of 16 slots in matrix-core operand order (:mod:`reinfer_amd.cache.layout`)."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+
+    def block_tensors(self, block_size: int):
+        from ..cache.layout import cache_shape
+        shape = cache_shape(1, self.num_kv_heads, block_size, self.head_dim)[1:]
+        return (("k", shape, None), ("v", shape, None))
 
 
 @dataclass(frozen=True)
@@ -26,10 +50,11 @@ class StateNeed:
 class LayerCache:
     """The cache of one run-order entry, as its mixer sees it.
 
-    For keys and values: ``k``/``v`` are ``[blocks, kv_heads, block_size // 16, 16 * head_dim]``,
-    tiles of 16 slots in the order of :mod:`reinfer_amd.cache.layout`;
-    ``group`` picks the step's block tables and slots, ``writes`` is False for an
-    entry that reads another entry's cache. For state: ``state`` is
+    Paged memory: ``tensors[name]`` is ``[blocks, *shape of one block]`` as the mixer's need named it;
+    for keys and values (:class:`KVNeed`) ``k``/``v`` are the same tensors,
+    ``[blocks, kv_heads, block_size // 16, 16 * head_dim]``, tiles of 16 slots in the order of
+    :mod:`reinfer_amd.cache.layout`; ``group`` picks the step's block tables and slots, ``writes`` is
+    False for an entry that reads another entry's cache. For state: ``state`` is
     ``[max_seqs, *shape]``, indexed by the step's ``state_slots``.
     """
     k: Optional[torch.Tensor] = None
@@ -37,6 +62,7 @@ class LayerCache:
     group: int = 0
     writes: bool = True
     state: Optional[torch.Tensor] = None
+    tensors: Optional[dict] = None      # every paged tensor by the name its mixer gave it ("k" and "v" among them)
 
 
 @dataclass

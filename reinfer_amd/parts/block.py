@@ -32,6 +32,10 @@ class PreNormBlock:
 
     def __init__(self, spec: BlockSpec, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
                  device: torch.device):
+        missing = [n for n in ("mixer", "ffn", "mixer_norm", "ffn_norm") if getattr(spec, n) is None]
+        if missing:
+            raise ValueError(f"a prenorm block is made of a mixer, a feed-forward and a norm before each; "
+                             f"block {spec.prefix!r} names no {', '.join(missing)}")
         p = spec.prefix
         self.spec = spec
         self.mixer_norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, weights,
@@ -42,6 +46,14 @@ class PreNormBlock:
         self.ffn = lookup("feed_forward", spec.ffn.kind)(spec.ffn, weights, p + spec.ffn_prefix, dtype, device)
 
     passes_emit = True      # forward(..., emit=) hands a NormTarget on to the feed-forward
+
+    def cache_need(self):
+        """What this layer keeps between steps: its mixer's need."""
+        return self.mixer.cache_need() if hasattr(self.mixer, "cache_need") else None
+
+    def parts(self):
+        """The parts this arrangement is made of (for whoever asks every part something)."""
+        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 
     def entry_target(self, resid: torch.Tensor):
         """A NormTarget for this block's first norm, for the part that runs before the block, or

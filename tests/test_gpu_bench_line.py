@@ -11,6 +11,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_bench_line_holds_the_contract():
+    """A test of the line's format: its keys, the flat configuration and the arithmetic between its figures. It
+    says nothing about whether the timed work is the model's (a bench that skipped work would pass it); that is
+    what the parity tests at these widths and ``check_run`` below are for."""
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "2", "--steps", "8", "--warmup", "4",
                         "--no-points", "--profile-steps", "1"], capture_output=True, text=True, timeout=600, cwd=ROOT)
     assert r.returncode == 0, r.stderr[-2000:]
@@ -41,3 +44,29 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120, cwd=ROOT)
     assert r.returncode == 2 and "one GPU" in (r.stdout + r.stderr)
+
+
+def test_bench_refuses_a_run_whose_results_are_not_a_models():
+    """``bench.check_run`` stands between every timed run and the line: logits that are not all finite, or a
+    request without tokens of the vocabulary, raise and nothing is printed."""
+    import torch
+    sys.path.insert(0, ROOT)
+    import bench
+    from helpers import TINY_A
+    from reinfer_amd.config import config_from_dict
+    from reinfer_amd.engine import LLMEngine
+    from reinfer_amd.sampling import SamplingParams
+    eng = LLMEngine(config=config_from_dict(TINY_A), seed=0, dtype="bfloat16", num_blocks=32)
+    for p in ([1, 2, 3, 4, 5], [7, 8, 9]):
+        eng.add_request(p, SamplingParams(temperature=0.0, max_tokens=50, ignore_eos=True))
+    for _ in range(4):
+        eng.step()
+    running = list(eng.scheduler.running)
+    bench.check_run(eng, TINY_A, running, "a good run")
+    eng.runner.last_logits[1, 17] = float("nan")
+    with pytest.raises(bench.InvalidRun, match="finite"):
+        bench.check_run(eng, TINY_A, running, "a bad run")
+    eng.step()
+    bench.check_run(eng, TINY_A, running, "the next step's logits are whole again")
+    with pytest.raises(bench.InvalidRun, match="vocabulary"):
+        bench.check_run(eng, dict(TINY_A, vocab_size=1), running, "tokens outside a vocabulary of one")

@@ -317,3 +317,21 @@ def test_decoding_requests_beside_two_prompt_portions_at_the_8b_widths(w8):
             runner.manager.check()
         finally:
             runner.poison_freed_blocks(False)
+
+
+def test_a_16384_token_prompt_in_one_step_at_the_32b_widths():
+    """The longest step the bench times: a 16,384-token prompt as one step through one layer of the Qwen3-32B
+    widths (64 query heads in groups of 8, so two workgroups a query tile and KV head; 256 query tiles; the
+    library's products and the row kernels at 16,384 rows), bfloat16, then a few tokens one by one behind
+    it. Logits at a spread of rows against the plain implementation."""
+    SHAPES["32b_long"] = dict(raw_config(1, 5120, 64, 25600, False), max_position_embeddings=16640)
+    w = Width("32b_long", max_tokens=16640, max_seqs=2)
+    try:
+        n = 16384 + 6
+        seqs = {"xxl": w.seq("xxl", n, 51)}
+        wanted = {"xxl": sorted({0, 1, 63, 64, 127, 128, 1000, 4095, 4096, 8191, 8192, 12000, 16319, 16320, 16382, 16383}
+                                | set(range(16384, n)))}
+        check(w, "bfloat16", seqs, [[("xxl", 16384)]] + [[("xxl", 1)]] * 6, wanted)
+    finally:
+        del w
+        torch.cuda.empty_cache()

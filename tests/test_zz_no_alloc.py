@@ -73,3 +73,42 @@ def test_sampling_without_allocation_refuses_what_the_array_cannot_hold():
     rc = lib.ra_sample_static(p, rows, vocab, vocab, p, p, p, p, ctypes.c_void_p(0))
     assert rc != 0
     assert b"scratch" in lib.ra_last_error()
+
+
+def test_sampling_without_allocation_inside_a_captured_stream():
+    """What the entry point is for: after ``ra_sample_static_prepare()`` (the address lookup, once, outside) it
+    is called while the stream captures, the graph is replayed several times with eager work between, each
+    replay on fresh logits, and every replay's tokens are those of ``ra_sample``; the device's free memory is the
+    same before and after the calls."""
+    from reinfer_amd.kernels import library
+    lib = library.load()
+    device = torch.device("cuda:0")
+    with torch.cuda.device(device):
+        assert lib.ra_sample_static_prepare() == 0, lib.ra_last_error()
+        rows, vocab = 12, 4099
+        logits, temperature, seeds, positions = _case(rows, vocab, 5, device)
+        got = torch.full((rows,), -9, dtype=torch.int32, device=device)
+        args = (ctypes.c_void_p(logits.data_ptr()), rows, vocab, logits.stride(0),
+                ctypes.c_void_p(temperature.data_ptr()), ctypes.c_void_p(seeds.data_ptr()),
+                ctypes.c_void_p(positions.data_ptr()), ctypes.c_void_p(got.data_ptr()))
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info(device)[0]
+        rc = lib.ra_sample_static(*args, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.ra_last_error()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(device)[0] == free_before, "an eager call changed the device's free memory"
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.ra_sample_static(*args, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.ra_last_error()
+        for rep in range(4):
+            fresh = _case(rows, vocab, 20 + rep, device)
+            for dst, src in zip((logits, temperature, seeds, positions), fresh):
+                dst.copy_(src)
+            got.fill_(-9)
+            graph.replay()
+            torch.cuda.synchronize()
+            want, eager = _both(lib, (logits, temperature, seeds, positions))     # eager work between the replays
+            assert torch.equal(got.cpu(), want), rep
+            assert torch.equal(eager, want)
