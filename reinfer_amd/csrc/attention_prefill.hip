@@ -164,11 +164,17 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     bf16x8_t kpre[NPRE], vpre[NPRE];
   };
   const int safe_kt = first_key & ~15;
+  // Which of the round's four tiles a thread fetches in step u: with two steps or more, neighbouring tiles (the
+  // two of a 32-key half), so that it holds both halves of every 16-byte piece of V's interleaved order and
+  // writes it whole (8-byte stores 32 bytes apart fall on a quarter of the LDS banks: measured, 23 % of the
+  // LDS's busy cycles were bank conflicts of those stores).
+  const int tile_group = __builtin_amdgcn_readfirstlane(tid / TCH);
+  auto tile_of = [&](int u) -> int { return NPRE >= 2 ? tile_group * NPRE + u : (tid + u * FP_THREADS) / TCH; };
+  const int w = tid % TCH;                         // the thread's 16-byte chunk of each of its tiles
   auto fetch = [&](Fetched& F, int k0) {
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
-      const int c = tid + u * FP_THREADS;
-      const int tt = __builtin_amdgcn_readfirstlane(c / TCH), w = c % TCH;
+      const int tt = __builtin_amdgcn_readfirstlane(tile_of(u));
       const int kt = k0 + tt * 16;
       const bool live = kt <= k_stop && kt + 15 >= first_key;           // wave-uniform
       const int ktl = live ? kt : safe_kt;
@@ -180,10 +186,10 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
     }
   };
   auto stage = [&](const Fetched& F, int k0, int buf) {
+    bf16x8_t vkeep = {0, 0, 0, 0, 0, 0, 0, 0};      // the even tile's values, until the odd tile's are there
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
-      const int c = tid + u * FP_THREADS;
-      const int tt = c / TCH, w = c % TCH;
+      const int tt = tile_of(u);
       const int kt = k0 + tt * 16;
       const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
       bf16x8_t kv = F.kpre[u], vv = F.vpre[u];
@@ -204,9 +210,18 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
         *(bf16x8_t*)(Ks2[buf] + (tt * 2 * d + w) * 8) = kv;
         // V: the two tiles of a half interleaved in runs of 8 bytes, so that an operand of the output
         // product (4 slots of the first tile, 4 of the second) is one 16-byte read
-        bf16_t* vd = Vs2[buf] + ((tt >> 1) * 4 * d + 2 * w) * 8 + (tt & 1) * 4;
-        *(bf16x4_t*)(vd) = (bf16x4_t){vv[0], vv[1], vv[2], vv[3]};
-        *(bf16x4_t*)(vd + 8) = (bf16x4_t){vv[4], vv[5], vv[6], vv[7]};
+        bf16_t* vd = Vs2[buf] + ((tt >> 1) * 4 * d + 2 * w) * 8;
+        if constexpr (NPRE >= 2) {
+          if (u & 1) {
+            *(bf16x8_t*)(vd) = (bf16x8_t){vkeep[0], vkeep[1], vkeep[2], vkeep[3], vv[0], vv[1], vv[2], vv[3]};
+            *(bf16x8_t*)(vd + 8) = (bf16x8_t){vkeep[4], vkeep[5], vkeep[6], vkeep[7], vv[4], vv[5], vv[6], vv[7]};
+          } else {
+            vkeep = vv;
+          }
+        } else {
+          *(bf16x4_t*)(vd + (tt & 1) * 4) = (bf16x4_t){vv[0], vv[1], vv[2], vv[3]};
+          *(bf16x4_t*)(vd + (tt & 1) * 4 + 8) = (bf16x4_t){vv[4], vv[5], vv[6], vv[7]};
+        }
       }
     }
   };
