@@ -576,6 +576,7 @@ struct Request {
   std::vector<int> output;
   int num_computed = 0;            // tokens of prompt + output whose keys are in the cache
   bool resumed = false;            // preempted at least once
+  bool aborted = false;
   py::object finish_reason = py::none();
   int preemptions = 0;
   // read once from params
@@ -612,7 +613,11 @@ using RequestP = std::shared_ptr<Request>;
 struct Portion {
   RequestP request;
   int start, length;
-  // the portion reaches the request's current end: its last logits give a token
+  // where in the request's output the token of this portion goes, once the step has been launched and
+  // until its token has been read (Scheduler::advance_blind / resolve); -1 otherwise
+  int out_index = -1;
+  // the portion reaches the request's current end: its last logits give a token (asked before the step is
+  // launched: afterwards the request has grown by the token's place)
   bool samples() const { return start + length == request->num_tokens(); }
 };
 
@@ -715,6 +720,7 @@ struct Scheduler {
       waiting.erase(std::find(waiting.begin(), waiting.end(), req));
     }
     req->state = FINISHED;
+    req->aborted = true;
     req->finish_reason = py::str("abort");
     forget(req);
     return true;
@@ -940,23 +946,67 @@ struct Scheduler {
   // The step ran: advance cursors, append sampled tokens, finish and free. Order of the checks:
   // stop ids, then the cap on new tokens, then the context (crates/scheduler/src/req.rs:281-314);
   // the stop token is consumed, not emitted.
-  std::vector<RequestP> complete(const StepPlan& plan, const py::dict& sampled) {
+  std::vector<RequestP> complete(StepPlan& plan, const py::dict& sampled) {
     std::vector<int> tokens;
     for (auto& p : plan.portions)
       if (p.samples()) tokens.push_back(sampled[p.request->rid].cast<int>());
     return complete_tokens(plan, tokens);
   }
   // The same with the sampled tokens as a list in the order of the portions that sample.
-  std::vector<RequestP> complete_tokens(const StepPlan& plan, const std::vector<int>& tokens) {
+  std::vector<RequestP> complete_tokens(StepPlan& plan, const std::vector<int>& tokens) {
+    advance_blind(plan);
+    return resolve(plan, tokens);
+  }
+
+  // The two halves of complete_tokens, for a caller that launches the next step before it has read this
+  // one's tokens. advance_blind: the step has been launched; cursors move, every request that samples
+  // grows by the place of its token (its value comes later), and what does not depend on the value is
+  // decided now: the cap on new tokens and the context end a request here, and its blocks go back at once
+  // (work queued on the GPU's stream before this moment is done before anything a later step launches).
+  // resolve: the tokens have been read; they take their places, and a token that stops its request (an
+  // end-of-sequence id, a stop id, the last of a stop sequence) cuts the output off before itself, together
+  // with whatever place a later step already added behind it: that step computed a row for a request that
+  // had ended, and the row is dropped. -> the requests whose end is known now, in the order of the portions.
+  static constexpr int TOKEN_PLACE = 0;        // what stands in an output until its token is read
+  void retire(const RequestP& r) {
+    if (r->state == RUNNING) {
+      running.erase(std::find(running.begin(), running.end(), r));
+      manager->free(r->rid);
+    } else if (r->state == WAITING) {            // preempted since: it holds nothing
+      auto it = std::find(waiting.begin(), waiting.end(), r);
+      if (it != waiting.end()) waiting.erase(it);
+    }
+    r->state = FINISHED;
+    ++c_finished;
+    forget(r);
+  }
+  void advance_blind(StepPlan& plan) {
+    for (auto& p : plan.portions) {
+      auto& r = p.request;
+      if (r->state != RUNNING) continue;         // aborted, or ended by an earlier token, since the plan was made
+      const bool samples = p.samples();          // before the cursor and the output move
+      r->num_computed = p.start + p.length;
+      if (!samples) continue;
+      p.out_index = (int)r->output.size();
+      r->output.push_back(TOKEN_PLACE);
+      if ((int)r->output.size() >= r->max_tokens || r->num_tokens() >= max_model_len) {
+        r->finish_reason = py::str("length");
+        retire(r);
+      }
+    }
+  }
+  std::vector<RequestP> resolve(StepPlan& plan, const std::vector<int>& tokens) {
     std::vector<RequestP> done;
     size_t next = 0;
     for (auto& p : plan.portions) {
-      auto& r = p.request;
-      const bool samples = p.samples();        // before the cursor and the output move
-      r->num_computed = p.start + p.length;
-      if (!samples) continue;
+      if (p.out_index < 0) continue;
       if (next >= tokens.size()) throw py::value_error("complete: fewer tokens than portions that sample");
       const int tok = tokens[next++];
+      auto& r = p.request;
+      const int idx = p.out_index;
+      p.out_index = -1;
+      if (r->aborted || idx >= (int)r->output.size()) continue;     // gone, or cut off by an earlier step's stop
+      r->output[idx] = tok;
       const bool is_eos = std::find(eos.begin(), eos.end(), tok) != eos.end();
       // A stop sequence fires the moment it is a suffix of the generated stream; its last token is
       // consumed like a stop id, the ones before it were emitted (crates/scheduler/src/stop.rs:1-12,
@@ -964,8 +1014,8 @@ struct Scheduler {
       bool seq_stop = false;
       for (auto& pat : r->stop_seqs) {
         const size_t L = pat.size();
-        if (tok != pat[L - 1] || r->output.size() + 1 < L) continue;
-        if (std::equal(pat.begin(), pat.end() - 1, r->output.end() - (L - 1))) {
+        if (tok != pat[L - 1] || (size_t)idx + 1 < L) continue;
+        if (std::equal(pat.begin(), pat.end() - 1, r->output.begin() + (idx + 1 - L))) {
           seq_stop = true;
           break;
         }
@@ -973,21 +1023,14 @@ struct Scheduler {
       const bool stop = seq_stop || (is_eos && !r->ignore_eos) ||
                         std::find(r->stop_ids.begin(), r->stop_ids.end(), tok) != r->stop_ids.end();
       if (stop) {
+        r->output.resize(idx);
         r->finish_reason = py::str("stop");
-      } else {
-        r->output.push_back(tok);
-        if ((int)r->output.size() >= r->max_tokens) r->finish_reason = py::str("length");
-        else if (r->num_tokens() >= max_model_len) r->finish_reason = py::str("length");
+        if (r->state != FINISHED) retire(r);     // (ended by the cap already: the stop wins, as it is checked first)
+      } else if (!(r->state == FINISHED && idx == (int)r->output.size() - 1)) {
+        continue;                                // goes on; or ended by the cap with a later token still to come
       }
-      if (!r->finish_reason.is_none()) {
-        r->state = FINISHED;
-        running.erase(std::find(running.begin(), running.end(), r));
-        manager->free(r->rid);
-        ++c_finished;
-        observe_output((long)r->output.size());
-        forget(r);
-        done.push_back(r);
-      }
+      observe_output((long)r->output.size());
+      done.push_back(r);
     }
     return done;
   }
@@ -1000,6 +1043,7 @@ struct Scheduler {
     std::vector<RequestP> rows;
     bool plain = true;
     for (auto& p : plan.portions) {
+      if (p.request->state != RUNNING) continue;      // ended by a token that was read after the plan was made
       auto e = std::make_shared<StepEntry>();
       e->rid = p.request->rid;
       e->tokens = p.request->tokens_slice(p.start, p.length);
@@ -1023,6 +1067,19 @@ struct Scheduler {
       sampling = py::make_tuple(temps, seeds, positions);
     }
     return py::make_tuple(entries, rows, sampling);
+  }
+
+  // Whether `next` is `prev` over again: the same requests in the same rows, one token each, every token drawn
+  // without a filter. Such a step can be launched before the tokens of `prev` have been read.
+  bool repeats(const StepPlan& prev, const StepPlan& next) const {
+    if (next.portions.empty() || next.portions.size() != prev.portions.size()) return false;
+    for (size_t i = 0; i < next.portions.size(); ++i) {
+      const Portion& p = next.portions[i];
+      if (p.request != prev.portions[i].request || p.length != 1 || !p.samples() || p.request->filters ||
+          p.request->state != RUNNING)
+        return false;
+    }
+    return true;
   }
 
   py::dict counters() const {
@@ -1191,5 +1248,8 @@ PYBIND11_MODULE(_host, m) {
       .def("schedule", &Scheduler::schedule)
       .def("entries_for", &Scheduler::entries_for, py::arg("plan"))
       .def("complete", &Scheduler::complete, py::arg("plan"), py::arg("sampled"))
-      .def("complete_tokens", &Scheduler::complete_tokens, py::arg("plan"), py::arg("tokens"));
+      .def("complete_tokens", &Scheduler::complete_tokens, py::arg("plan"), py::arg("tokens"))
+      .def("advance_blind", &Scheduler::advance_blind, py::arg("plan"))
+      .def("repeats", &Scheduler::repeats, py::arg("prev"), py::arg("next"))
+      .def("resolve", &Scheduler::resolve, py::arg("plan"), py::arg("tokens"));
 }

@@ -152,11 +152,16 @@ class _CapturedStep:
             self.copied.synchronize()
         self.rows.fill(entries, self.h, sampling)
 
-    def replay(self) -> None:
+    def replay(self, token_source: Optional[torch.Tensor] = None) -> None:
         self.dev.copy_(self.host, non_blocking=True)
         if self.copied is None:
             self.copied = torch.cuda.Event()
         self.copied.record()
+        if token_source is not None:
+            # the step's tokens are those that the step before it drew, still on the device: they take the
+            # place of what the host wrote (it does not know them yet)
+            n = token_source.numel()
+            self.batch.token_ids[:n].copy_(token_source, non_blocking=True)
         self.graph.replay()
 
 
@@ -167,10 +172,12 @@ class DecodeGraphs:
         self.pool = None
         self.replays = 0
 
-    def run(self, entries: List[StepEntry], longest: int, sampling=None):
+    def run(self, entries: List[StepEntry], longest: int, sampling=None, token_source: Optional[torch.Tensor] = None):
         """A step of at most MAX_GRAPH_BATCH entries with one token each; ``longest`` is the longest
         context after it. -> (logits [B_pad, vocab] static, tokens [B_pad] static): rows past the
-        entries are padding; both are overwritten by the next replay of this bucket."""
+        entries are padding; both are overwritten by the next replay of this bucket. ``token_source``: an
+        int32 device tensor, one token per entry, that replaces the entries' own tokens (the tokens of the
+        step before, which the host has not read yet)."""
         r = self.runner
         B = _batch_bucket(len(entries))
         # context buckets are powers of two from 256, and never more than the block tables hold (a
@@ -185,6 +192,6 @@ class DecodeGraphs:
             cs = _CapturedStep(r, B, ctx_cap, self.pool)
             self.steps[key] = cs
         cs.fill(entries, sampling)
-        cs.replay()
+        cs.replay(token_source)
         self.replays += 1
         return cs.logits, cs.tokens

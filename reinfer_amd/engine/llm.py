@@ -62,6 +62,10 @@ class LLMEngine:
                                    max_model_len=self.runner.max_model_len, max_chunk=max_chunk,
                                    eos_token_ids=self.runner.spec.eos_token_ids, admission=admission)
         self.sampler = Sampler(self.device)
+        self._pending = None        # the step launched last: (plan, requests that sample, device tokens, host tokens, event)
+        pin = self.device.type == "cuda"
+        self._token_buffers = [torch.zeros(max(1, int(max_num_seqs)), dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._token_turn = 0
         self._auto_id = 0
         self.timings: Dict[str, float] = {}
 
@@ -85,33 +89,90 @@ class LLMEngine:
         return self.scheduler.abort(rid)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._pending is not None
 
     # -------------------------------------------------------------- step
+    # A step is launched in one call and its tokens are read in the next: between the two the scheduler
+    # has advanced every request by the place of its token (``advance_blind``) and plans the step after it
+    # without the token's value. Where that next step is the same requests decoding again, it is launched
+    # at once, its tokens handed over on the device (the captured step's input buffer is filled from the
+    # sampler's output buffer), and only then are the earlier step's tokens read: the GPU goes from one
+    # decode step to the next without waiting for the host. A request that a token ended (an end-of-sequence
+    # or stop id) has by then one more row in flight; the row is dropped (``resolve``). What the scheduler
+    # assumes: whether a request goes on after a step does not depend on the step's token, until it is told
+    # otherwise one step later; so a request ended by a token leaves one step later than it might, and a
+    # waiting request takes its place one step later. Tokens do not depend on any of this: a request's
+    # noise is a function of its seed and position.
     def step(self) -> List[RequestOutput]:
-        """One scheduler decision, one batch through the model, one sampling call."""
+        """One scheduler decision and one batch launched; the tokens of the batch launched by the call
+        before are read, and the requests they ended are returned."""
+        pending = self._pending
         plan = self.scheduler.schedule()
         finished = [self._output(r) for r in plan.finished]
-        if not plan.portions:
-            if not finished and self.scheduler.has_work() and not plan.preempted:
-                raise RuntimeError("the scheduler could place no token although work is waiting")
+        if pending is None:
+            if not plan.portions:
+                if not finished and self.scheduler.has_work() and not plan.preempted:
+                    raise RuntimeError("the scheduler could place no token although work is waiting")
+                return finished
+            self._launch(plan, None)
             return finished
-        # entries as the step takes them; where every entry wants one token and none shapes its
-        # distribution, the step may draw the tokens itself
+        if plan.portions and self._chains(pending, plan):
+            self._launch(plan, pending)
+            done = self._resolve(pending)
+        else:
+            # the next step needs tokens the host has to see first (a prompt's first token, a row that a
+            # filter shapes), or is another set of rows: read, then launch
+            done = self._resolve(pending)
+            self._pending = None
+            if plan.portions:
+                self._launch(plan, None)
+            elif not finished and not done and self.scheduler.has_work() and not plan.preempted:
+                raise RuntimeError("the scheduler could place no token although work is waiting")
+        return finished + [self._output(r) for r in done]
+
+    def _chains(self, pending, plan: StepPlan) -> bool:
+        """The planned step is the one just launched over again: the same requests, one token each, all
+        drawn inside the captured step."""
+        return pending[2] is not None and self.runner.can_chain(len(pending[1])) \
+            and self.scheduler.repeats(pending[0], plan)
+
+    def _launch(self, plan: StepPlan, chained_from) -> None:
+        # a request that an earlier token ended since the plan was made has no part in the step
         entries, rows, sampling = self.scheduler.entries_for(plan)
-        logits, toks = self.runner.step_sampled(entries, sampling)
+        if not entries:
+            self._pending = None
+            return
+        if chained_from is not None:
+            logits, toks = self.runner.step_sampled(entries, sampling, token_source=chained_from[2][:len(rows)])
+        else:
+            logits, toks = self.runner.step_sampled(entries, sampling)
+        tokens_host = event = None
         if toks is not None:
-            out = toks.tolist()
-            if min(out) < 0:
+            # out of the step's own buffer (the next replay overwrites it) into pinned memory, without waiting
+            tokens_host = self._token_buffers[self._token_turn][:len(rows)]
+            self._token_turn ^= 1
+            tokens_host.copy_(toks, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        elif rows:
+            tokens_host = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
+                                              [r.num_tokens for r in rows], [r.tokens for r in rows])
+        else:
+            tokens_host = []
+        self.scheduler.advance_blind(plan)
+        self._pending = (plan, rows, toks, tokens_host, event)
+
+    def _resolve(self, pending) -> List[Request]:
+        plan, rows, _, tokens_host, event = pending
+        if event is not None:
+            event.synchronize()
+            out = tokens_host.tolist()
+            if out and min(out) < 0:
                 r = rows[[t < 0 for t in out].index(True)]
                 raise SamplingError(f"request {r.rid!r}: no finite logit to sample from")
-        elif rows:
-            out = self.sampler.sample(logits, [r.params for r in rows], [r.seed for r in rows],
-                                      [r.num_tokens for r in rows], [r.tokens for r in rows])
         else:
-            out = []
-        done = self.scheduler.complete_tokens(plan, out)
-        return finished + [self._output(r) for r in done]
+            out = list(tokens_host)
+        return self.scheduler.resolve(plan, out)
 
     @staticmethod
     def _output(r: Request) -> RequestOutput:
@@ -133,7 +194,7 @@ class LLMEngine:
         outs: Dict[Hashable, RequestOutput] = {}
         t0 = time.perf_counter()
         first = None
-        while self.scheduler.has_work():
+        while self.has_unfinished():
             for o in self.step():
                 outs[o.rid] = o
             if first is None:

@@ -237,19 +237,30 @@ class ModelRunner:
         and behind every layer (such a step never replays a captured graph)."""
         return self.step_sampled(entries, None, observer)[0]
 
-    def step_sampled(self, entries: Sequence[StepEntry], sampling=None, observer=None):
+    def can_chain(self, n_entries: int) -> bool:
+        """Whether a step of ``n_entries`` single tokens can take its tokens from the device (``token_source``)."""
+        return self.graphs is not None and 0 < n_entries <= MAX_GRAPH_BATCH
+
+    def step_sampled(self, entries: Sequence[StepEntry], sampling=None, observer=None, token_source=None):
         """As :meth:`step`; ``sampling`` = (temperatures, seeds, positions), one per entry,
         asks for a token from each entry's single wanted row where the step can draw it
         itself. -> (logits, tokens): ``tokens`` is an int32 device tensor, one per
-        entry, or None when the caller has to sample from the logits."""
+        entry, or None when the caller has to sample from the logits. ``token_source`` (only for a step
+        of single tokens that replays a captured graph, see :meth:`can_chain`): the entries' tokens are
+        taken from this device tensor, not from the entries."""
         if not isinstance(entries, list):
             entries = list(entries)
+        if token_source is not None and not (self.can_chain(len(entries)) and observer is None
+                                             and all(len(e.tokens) == 1 for e in entries)):
+            raise ValueError("token_source: only a step of single tokens that replays a captured graph takes its "
+                             "tokens from the device")
         # checks every entry (StepError), then takes the blocks of all of them or raises OutOfBlocks
         one_token, one_want, longest = self.manager.begin_step(entries, self.spec.vocab_size,
                                                                self.max_model_len)
         tokens = None
-        if self.graphs is not None and one_token and len(entries) <= MAX_GRAPH_BATCH and observer is None:
-            all_logits, all_tokens = self.graphs.run(entries, longest, sampling)
+        graphed = self.graphs is not None and one_token and len(entries) <= MAX_GRAPH_BATCH and observer is None
+        if graphed:
+            all_logits, all_tokens = self.graphs.run(entries, longest, sampling, token_source)
             n = len(entries)
             if one_want:
                 logits = all_logits[:n]

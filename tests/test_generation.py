@@ -221,3 +221,28 @@ def test_aborts_and_arrivals_between_captured_decode_steps(tmp_path):
     assert {k: outs[k].token_ids for k in outs} == {k: alone[k] for k in outs}
     assert eng.runner.graphs is not None and eng.runner.graphs.replays > 30
     assert eng.cache_stats()["blocks_free"] == eng.cache_stats()["blocks_total"]
+
+
+@pytest.mark.gpu
+def test_a_token_that_ends_a_request_is_read_one_step_late(tmp_path):
+    """Decode steps are launched before the tokens of the step before have been read: a request that its
+    end-of-sequence id ended has one more row in flight by then. Several requests decode together, the id ends
+    them at different steps: each has the tokens of the plain loop up to (not including) the id, the others go
+    on undisturbed, every block comes back."""
+    folder = make_folder(tmp_path, "A", "float32")
+    raw, w = read_folder(folder)
+    prompts = [random_tokens(n, raw["vocab_size"], 60 + n) for n in (6, 11, 19, 4)]
+    free = [plain.greedy_generate(raw, w, p, 14) for p in prompts]
+    eos = free[0][3]
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(dict(raw, eos_token_id=eos), f)
+    eng = engine_for(folder, "cuda:0", num_blocks=32)
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=14))
+    for run, o in zip(free, outs):
+        want = run[:run.index(eos)] if eos in run else run
+        assert o.token_ids == want
+        assert o.finish_reason == ("stop" if eos in run else "length")
+    assert outs[0].finish_reason == "stop" and any(o.finish_reason == "length" for o in outs)
+    assert eng.runner.graphs is not None and eng.runner.graphs.replays >= 10
+    assert eng.cache_stats()["blocks_free"] == eng.cache_stats()["blocks_total"]
+    assert not eng.has_unfinished()

@@ -366,3 +366,79 @@ def test_finished_requests_are_forgotten():
     assert all(r.state == FINISHED and len(r.output) == 3 for r in held)     # the caller's objects live on
     s.add("r0", [1, 2, 3], SamplingParams(max_tokens=1), seed=0)             # an id may be used again
     assert set(drive(m, s)) == {"r0"}
+
+
+def drive_one_step_late(m, s, token_fn=fake_token, aborts=None, limit=10000):
+    """The loop of the engine that launches a step before it has read the tokens of the step before:
+    schedule, launch (here: take the blocks), advance blind, and only then resolve the step before."""
+    outs, pending, n = {}, None, 0
+    aborts = dict(aborts or {})
+    while s.has_work() or pending is not None:
+        plan = s.schedule()
+        for r in plan.finished:
+            outs[r.rid] = (list(r.output), r.finish_reason)
+        live = [p for p in plan.portions if p.request.state == RUNNING]
+        for p in live:
+            assert p.start == p.request.num_computed
+            m.grow(p.request.rid, p.start + p.length)
+        for p in live:
+            m.commit(p.request.rid, p.start + p.length)
+        tokens = [token_fn(p.request.rid, p.request.num_tokens) for p in live if p.samples]
+        s.advance_blind(plan)
+        if pending is not None:
+            for r in s.resolve(*pending):
+                outs[r.rid] = (list(r.output), r.finish_reason)
+        pending = (plan, tokens) if live else None
+        for rid in aborts.pop(n, []):
+            s.abort(rid)
+        m.check()
+        n += 1
+        assert n < limit, "the scheduler does not terminate"
+    return outs
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_tokens_read_one_step_late_change_nothing(seed):
+    """Requests whose tokens are read a step late (the next step is planned and launched first) end with the
+    tokens and reasons of the loop that reads at once: a stop token cuts off the place that the later step
+    had already added, the cap and the context end a request at launch time, a stop at the very last token
+    still wins over the cap; under preemptions (a pool too small for all) and with stop sequences."""
+    import random
+    rng = random.Random(seed)
+    reqs = []
+    for i in range(14):
+        stops = ([rng.randrange(20)] if rng.random() < 0.5 else [])
+        seqs = ([[rng.randrange(20), rng.randrange(20)]] if rng.random() < 0.4 else [])
+        reqs.append((f"r{i}", [rng.randrange(1000) for _ in range(rng.randrange(1, 40))],
+                     SamplingParams(max_tokens=rng.randrange(1, 30), stop_token_ids=stops, stop_sequences=seqs)))
+
+    def tok(rid, position):
+        return fake_token(rid, position, vocab=20)          # few values: stops and stop sequences do fire
+
+    results = []
+    for driver in (drive, drive_one_step_late):
+        m, s = make(num_blocks=30, bs=4, max_seqs=5, budget=24, max_chunk=12, eos=(7,), max_model_len=60)
+        for rid, prompt, params in reqs:
+            s.add(rid, prompt, params, seed=0)
+        outs = driver(m, s, token_fn=tok)
+        assert all(p.num_free == p.num_blocks for p in m.pools)
+        assert not s.running and not s.waiting
+        results.append((outs, s.counters["preemptions"]))
+    assert results[0][0] == results[1][0]
+    reasons = {r for _, r in results[0][0].values()}
+    assert {"stop", "length"} <= reasons, reasons
+
+
+def test_abort_and_stop_while_a_step_is_in_flight():
+    m, s = make(num_blocks=40, bs=4, eos=(5,))
+    for i in range(3):
+        s.add(f"r{i}", [1, 2, 3], SamplingParams(max_tokens=20), seed=0)
+    # r1's second token is the end-of-sequence id; r2 is aborted while a step with its row is in flight
+    def tok(rid, position):
+        return 5 if (rid, position) == ("r1", 4) else 100 + position
+    outs = drive_one_step_late(m, s, token_fn=tok, aborts={2: ["r2"]})
+    assert outs["r1"] == ([103], "stop")
+    assert outs["r0"][1] == "length" and outs["r0"][0] == [100 + p for p in range(3, 23)]
+    assert "r2" not in outs                     # an aborted request is not reported as done
+    assert all(p.num_free == p.num_blocks for p in m.pools)
+    assert s.counters["finished"] == 2
