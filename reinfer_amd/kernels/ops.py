@@ -223,7 +223,11 @@ class HipKernels:
         # query tiles that give every CU one workgroup
         room = self._cus(q.device) // max(1, lib.ra_attention_prefill_groups(num_heads, num_kv_heads, head_dim))
         halves = lib.ra_attention_prefill_columns(num_heads, num_kv_heads, head_dim) == 2
-        plan = self._attention_plan(batch, q.device, tile, room, halves)
+        # the plan's fixed costs are priced in rounds of this shape: a round's time goes with the columns of a
+        # query tile times the head size the kernel is built for
+        cols = 128 * max(1, lib.ra_attention_prefill_columns(num_heads, num_kv_heads, head_dim))
+        built_for = 64 if head_dim <= 64 else 128 if head_dim <= 128 else 256
+        plan = self._attention_plan(batch, q.device, tile, room, halves, (256 * 128) / (cols * built_for))
         dec_ok = bool(lib.ra_attention_decode_supports(num_heads, num_kv_heads, head_dim, bs))
         pre_ok = bool(lib.ra_attention_prefill_supports(num_heads, num_kv_heads, head_dim, bs))
         side = None
@@ -271,10 +275,11 @@ class HipKernels:
             n = self._cu_count[device] = int(torch.cuda.get_device_properties(device).multi_processor_count)
         return n
 
-    # What the prompt kernel's plan is chosen by, in rounds of 64 keys of a whole query tile (2.1 us with 32
-    # heads of 128 over 8 groups): a tile listed with half of its heads costs 0.76 of the whole one, every
-    # listed item one round to start and end, and the kernel that adds the parts of cut tiles 3 rounds and
-    # 0.15 for each part (measured: a portion of 512 tokens behind 3584: 142 us as it is, 115 with the tiles
+    # What the prompt kernel's plan is chosen by, in rounds of 64 keys of a whole query tile of 256 columns
+    # and head size 128 (2.1 us: 64 queries of 4 heads): a tile listed with half of its heads costs 0.76 of the
+    # whole one, every listed item one such round to start and end, and the kernel that adds the parts of cut
+    # tiles 3 rounds and 0.15 for each part; for another shape the three fixed costs are scaled by how much
+    # shorter or longer its rounds are (``fixed``: the reference round's work over this shape's) (measured: a portion of 512 tokens behind 3584: 142 us as it is, 115 with the tiles
     # listed twice, 57 cut by keys; 256 behind 7936: 277 / 223 / 58; a whole prompt of 2048: 83 / 69 / 83,
     # of 1024: 43 / 35 / 40; 2048 behind 2048: 152 / 195 / 146)
     PREFILL_ROUND = 64
@@ -297,7 +302,7 @@ class HipKernels:
             heapq.heappush(ends, heapq.heappop(ends) + c)
         return max(ends)
 
-    def _prefill_items(self, tiles, room: int, halves: bool):
+    def _prefill_items(self, tiles, room: int, halves: bool, fixed: float = 1.0):
         """The prompt kernel's work items for ``tiles`` of (request, row, queries, position), and the list
         for the kernel that adds the parts of tiles cut by keys: ``(items, merge, n_slots)``, an item being
         (cost, tile, first key, one past the last key, slot or -1).
@@ -316,8 +321,9 @@ class HipKernels:
         layer's window finds nothing to do.)"""
         R = self.PREFILL_ROUND
         n = len(tiles)
+        item_cost = self.PREFILL_ITEM * fixed
         rounds = [-(-(pos + q) // R) for (_, _, q, pos) in tiles]
-        whole = [(r + self.PREFILL_ITEM, tl, 0, 0, -1) for tl, r in zip(tiles, rounds)]
+        whole = [(r + item_cost, tl, 0, 0, -1) for tl, r in zip(tiles, rounds)]
         if room <= 0 or n == 0:
             return whole, [], 0
         best, best_span = (whole, [], 0), self._span([it[0] for it in whole], room)
@@ -335,7 +341,7 @@ class HipKernels:
             for k, (tl, r) in enumerate(zip(tiles, rounds)):
                 if k in twice:
                     i, row, q, pos = tl
-                    c = r * self.PREFILL_HALF_HEADS + self.PREFILL_ITEM
+                    c = r * self.PREFILL_HALF_HEADS + item_cost
                     items.append((c, (i, row, q | (1 << 16), pos), 0, 0, -1))
                     items.append((c, (i, row, q | (2 << 16), pos), 0, 0, -1))
                 else:
@@ -366,11 +372,11 @@ class HipKernels:
                 merge.extend((tl[1], tl[2], n_slots, p))
                 for j in range(p):
                     hi = (j + 1) * per * R if j + 1 < p else 1 << 30
-                    items.append((min(per, r - j * per) + self.PREFILL_ITEM, tl, j * per * R, hi, n_slots + j))
+                    items.append((min(per, r - j * per) + item_cost, tl, j * per * R, hi, n_slots + j))
                 n_slots += p
             if n_slots:
-                span = self._span([it[0] for it in items], room) + self.PREFILL_MERGE[0] \
-                    + self.PREFILL_MERGE[1] * n_slots
+                span = self._span([it[0] for it in items], room) + (self.PREFILL_MERGE[0]
+                                                                      + self.PREFILL_MERGE[1] * n_slots) * fixed
                 if span < best_span:
                     best, best_span = (items, merge, n_slots), span
         return best
@@ -382,14 +388,14 @@ class HipKernels:
             "n_decode": num_rows, "decode_max_ctx": ctx_cap, "decode_list": None, "n_prefill": 0,
             "prefill_list": None, "n_tiles": 0, "tiles": None}
 
-    def _attention_plan(self, batch, device, tile: int, room: int = 0, halves: bool = False):
+    def _attention_plan(self, batch, device, tile: int, room: int = 0, halves: bool = False, fixed: float = 1.0):
         """Which tokens go to which kernel; made once per step and query-tile size, shared by the
         layers. ``room`` is the number of query tiles whose workgroups fill the chip once (0: the tiles
         are listed as they are)."""
         plan = batch.extra.get("attention_plan")
         if plan is not None and plan.get("tile", tile) == tile:
             return plan
-        plan = batch.extra.get(("attention_plan", tile, room, halves))
+        plan = batch.extra.get(("attention_plan", tile, room, halves, fixed))
         if plan is not None:
             return plan
         dec, pre, tiles = [], [], []
@@ -404,7 +410,7 @@ class HipKernels:
                 for q0 in range(0, ql, tile):
                     tiles.append((i, t + q0, min(tile, ql - q0), st + q0))
             t += ql
-        items, merge, n_slots = self._prefill_items(tiles, room, halves)
+        items, merge, n_slots = self._prefill_items(tiles, room, halves, fixed)
         items.sort(key=lambda it: it[0])                     # the heaviest last: the kernel starts the last listed first
         listed = [v for it in items for v in it[1]]
         ranges = [v for it in items for v in ((it[2], it[3], it[4]) if it[4] >= 0 else (0, 1 << 30, -1))] if merge else []
@@ -427,7 +433,7 @@ class HipKernels:
             "n_merge": len(merge) // 4, "n_slots": n_slots,
             "tile": tile,
         }
-        batch.extra[("attention_plan", tile, room, halves)] = plan
+        batch.extra[("attention_plan", tile, room, halves, fixed)] = plan
         return plan
 
     @staticmethod
@@ -476,7 +482,7 @@ class HipKernels:
     # 10.6 / 13.1 / 23.3 / 40.4 / 61.3 / 107 us, 12 waves 13.6 / 14.5 / 21.5 / 33.8 / 56.2 / 107; 8000 keys,
     # 1 / 4 / 16 / 64 tokens: 17.9 / 35.9 / 113 / 370 against 14.7 / 31.2 / 101 / 364)
     DECODE_WIDE_PAIRS = 64
-    DECODE_WIDE_CTX = 4096
+    DECODE_WIDE_CTX = 4096      # keys of head size 128: what counts is the bytes of a (token, KV head) pair
 
     def _slots_of_decode(self, num_heads: int, num_kv_heads: int, head_dim: int, waves: int) -> int:
         """Workgroups of the decode kernel's form with ``waves`` waves that the chip holds at once (0: that
@@ -503,7 +509,7 @@ class HipKernels:
         a CU)."""
         pairs = max(1, n_tokens * num_kv_heads)
         waves = 4
-        if pairs >= self.DECODE_WIDE_PAIRS or max_ctx > self.DECODE_WIDE_CTX:
+        if pairs >= self.DECODE_WIDE_PAIRS or max_ctx * head_dim > self.DECODE_WIDE_CTX * 128:
             wide = self._slots_of_decode(num_heads, num_kv_heads, head_dim, 12)
             # whole rounds of the large workgroups, or nearly (64 requests over 8 KV heads are two rounds
             # of 256: 8.45 ms a step against 8.65 with the small workgroups)

@@ -124,15 +124,16 @@ def run_plan(runner, seqs: Dict[str, Sequence[int]], plan, ends=None, want_all: 
 
 
 def mixed_plan():
-    """Five requests, at most four live, portions beside single tokens, 160 tokens of cache."""
-    lens = {"a": 40, "b": 33, "c": 50, "d": 29, "e": 47}
+    """Six requests, four of them live in the third step, portions beside single tokens, 128 tokens of cache:
+    the four that are live together fill all eight blocks of 16 between them, and the requests that come
+    after them run on blocks that were given back."""
+    lens = {"a": 30, "b": 20, "c": 30, "d": 20, "e": 40, "f": 25}
     plan = [
         [("a", 9), ("b", 2)],
-        [("a", 1), ("b", 20), ("c", 5)],
-        [("a", 30), ("b", 1), ("c", 1)],
-        [("b", 10), ("c", 44)],
-        [("d", 27), ("e", 3)],
-        [("d", 1), ("e", 43)],
-        [("d", 1), ("e", 1)],
+        [("a", 1), ("b", 17), ("c", 5)],
+        [("a", 20), ("b", 1), ("c", 12), ("d", 17)],
+        [("c", 13), ("d", 3), ("e", 3)],
+        [("e", 36), ("f", 2)],
+        [("e", 1), ("f", 23)],
     ]
     return lens, plan
