@@ -75,7 +75,6 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   const int kb = blockIdx.y * k_per_split;
   const int ke = min(K, kb + k_per_split);
   const int n_runs = (ke - kb + GW_KS - 1) / GW_KS;
-  const int n_runs_p = (n_runs + GW_DEPTH - 1) / GW_DEPTH * GW_DEPTH;      // padded with runs of zeros
   bf16_t* my_w = lds_w + wave * WTILE;
 
   // Both operands are read through buffer descriptors: a load whose offset lies past the descriptor's
@@ -184,10 +183,17 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
       }
     }
   }
-  for (int run = 0; run < n_runs_p; run += GW_DEPTH) {  // the same in every thread of the workgroup
+  // Whole groups of GW_DEPTH runs in the loop, the runs left over behind it: padding the range with runs of
+  // zeros instead costs a short range half as much again (four runs became six), and a condition out here
+  // costs the loop's waits nothing. The loads that a step asks for past the range's end are out as a whole.
+  const int n_whole = n_runs / GW_DEPTH * GW_DEPTH;
+  for (int run = 0; run < n_whole; run += GW_DEPTH) {  // the same in every thread of the workgroup
 #pragma unroll
     for (int d = 0; d < GW_DEPTH; ++d) step(R[d], run + d);
   }
+#pragma unroll
+  for (int d = 0; d < GW_DEPTH - 1; ++d)
+    if (n_whole + d < n_runs) step(R[d], n_whole + d);
   if (EPI != WEPI_PARTIAL && nf.in_ss) {
     // first touched here: an empty volatile statement per value keeps the compiler from moving
     // arithmetic on it, and with it the wait for it, up in front of the loop
@@ -321,8 +327,8 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
 
 // How [M, N, K] is cut: waves a workgroup (5 to 8, 16 features each) and K ranges. With many features
 // one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
-// workgroups of 96; 19456: 244 of 80; 51200: 458 of 112). With few features 128 a workgroup and the smallest power of two up to 8 of K
-// ranges that gives at least three quarters as many workgroups as the chip has CUs (192 of 256), each range a multiple of the run and two runs or more.
+// workgroups of 96; 19456: 244 of 80; 51200: 458 of 112). With few features 128 a workgroup and as many K ranges as
+// give one workgroup a CU or fewer, each range a multiple of the run.
 static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int* k_per_split, bool* partial = nullptr,
                      bool emits = false) {
   if (partial) *partial = emits;                       // the adding kernel writes what the next norm needs
@@ -351,8 +357,14 @@ static void gw_split(int epilogue, int M, int N, int K, int* waves, int* S, int*
     }
     return;
   }
-  int s = 1;
-  while (s < 8 && cb8 * s < fill && K / (s * 2) >= 2 * GW_KS) s *= 2;
+  // As many ranges as fill the chip's CUs once and no more: workgroups of a second, part-filled round last as
+  // long as those of the first (64 rows, 10240 x 5120: 4 ranges, 320 workgroups, 34 us; 3 ranges, 240
+  // workgroups, 26 us; 5120 x 25600: 8 ranges 77 us, 6 ranges 55 us). A range is four runs or more (shorter
+  // ones are all start and end), and there are at most 12 (each is a float plane to write and read again).
+  int s = cus / cb8;
+  if (s > 12) s = 12;
+  while (s > 1 && K / s < 4 * GW_KS) --s;
+  if (s < 1) s = 1;
   int kps = (K + s - 1) / s;
   kps = (kps + GW_KS - 1) / GW_KS * GW_KS;
   *S = (K + kps - 1) / kps;
