@@ -255,8 +255,15 @@ __global__ void qk_norm_rope_cache_kernel(TA* __restrict__ qkv, const TW* __rest
       }
       const float* src = sm.parts + ((size_t)t * n_heads + head) * d;
       for (int i = lane; i < d; i += RA_WAVE) {
-        float v = 0.f;
-        for (int r = 0; r < sm.n_ranges; ++r) v += src[(size_t)r * sm.range_stride + i];        // range order
+        float v = 0.f;                         // range order; six ranges' values asked for in one trip
+        constexpr int U = 6;
+        for (int r0 = 0; r0 < sm.n_ranges; r0 += U) {
+          float tv[U];
+#pragma unroll
+          for (int j = 0; j < U; ++j) tv[j] = src[(size_t)min(r0 + j, sm.n_ranges - 1) * sm.range_stride + i];
+#pragma unroll
+          for (int j = 0; j < U; ++j) v += r0 + j < sm.n_ranges ? tv[j] : 0.f;
+        }
         v *= row;
         b[i] = v;
         ss += v * v;

@@ -286,13 +286,23 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (n < N) {
     const bool whole = n + 3 < N && (N & 3) == 0;
-    for (int s = 0; s < S; ++s) {
-      const float* p = P + ((size_t)s * M + m) * N + n;
-      if (whole) {
-        const f32x4_t t = *(const f32x4_t*)p;
+    if (whole) {
+      // six ranges' values are asked for in one trip and then added in range order (one by one, the loop
+      // made a trip a range)
+      constexpr int U = 6;
+      for (int s0 = 0; s0 < S; s0 += U) {
+        f32x4_t t[U];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] += t[i];
-      } else {
+        for (int j = 0; j < U; ++j)
+          t[j] = *(const f32x4_t*)(P + ((size_t)min(s0 + j, S - 1) * M + m) * N + n);
+#pragma unroll
+        for (int j = 0; j < U; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] += s0 + j < S ? t[j][i] : 0.f;
+      }
+    } else {
+      for (int s = 0; s < S; ++s) {
+        const float* p = P + ((size_t)s * M + m) * N + n;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (n + i < N) v[i] += p[i];

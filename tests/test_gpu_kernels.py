@@ -235,7 +235,8 @@ def test_qk_norm_rope_cache_values_of_four_slots_in_a_row(dtype, Hq, Hkv, d):
 
 @pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [(4, 2, 16, 16, 0, True), (3, 1, 80, 32, 0, False),
                                                       (6, 3, 64, 64, 1, True), (32, 8, 128, 128, 0, True)])
-@pytest.mark.parametrize("T,S,carried", [(5, 1, False), (33, 4, True), (64, 3, True), (20, 2, False)])
+@pytest.mark.parametrize("T,S,carried", [(5, 1, False), (33, 4, True), (64, 3, True), (20, 2, False), (40, 6, True),
+                                         (18, 7, False), (64, 11, True)])
 def test_qk_norm_rope_cache_from_the_ranges_of_a_split_product(Hq, Hkv, d, rot, style, norm, T, S, carried):
     """The same kernel fed with the float results of the K ranges of a split product, which it adds
     itself, and with the partial sums of squares of an RMSNorm carried by that product: equal to
