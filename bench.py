@@ -366,7 +366,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points and the further sizes")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1, 64 and 128 points and the further sizes")
     ap.add_argument("--no-profile", action="store_true", help="skip the per-kernel-class times of the decode step")
     ap.add_argument("--profile-steps", type=int, default=4, help="decode steps timed kernel by kernel")
     ap.add_argument("--seed", type=int, default=0)
@@ -401,7 +401,7 @@ def main() -> int:
         return serve_run(args, raw, shape_name)
     cfg = config_from_dict(raw)
     ctx_len = raw["max_position_embeddings"]
-    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_batch = max(args.batch, 1 if args.no_points else 128)
     block = 16
     # a request decodes while later prompts are still being prefilled: one step a portion of a prompt
     budget = max(2048, args.prefill_tokens)
@@ -446,8 +446,8 @@ def main() -> int:
 
     points, fracs, serve = {}, {}, None
     if not args.no_points:
-        for b in (1, 64):
-            steps_b = args.steps if b == 1 else max(16, args.steps // 2)
+        for b in (1, 64, 128):
+            steps_b = args.steps if b == 1 else max(16, args.steps // (2 if b == 64 else 4))
             pms, pctx = decode_run(engine, raw, b, args.prompt_len, steps_b, min(args.warmup, 16), args.seed + 3 + b, max_new)
             points[f"decode_b{b}"] = round(b / (pms * 1e-3), 1)
             fracs[f"decode_b{b}"] = round((n_lin * elem + b * pctx * kv_tok) / (pms * 1e-3) / HBM_PEAK, 4)

@@ -396,7 +396,9 @@ extern "C" int ra_gemm_wide_preferred(int epilogue, int M, int N, int K) {
   // 65 to 128 rows: the library's products are as fast or faster (151936 x 4096 at 128 rows: 285 us against
   // 400) but for a product that adds into the residual stream over a long K, which this kernel cuts into
   // ranges (4096 x 12288 at 96 / 128 rows: 37 / 43 us against 59 / 70 for the library's product and the add)
-  if (M > 64) return (epilogue == WEPI_ACCUM && S > 1 && large) ? 1 : 0;
+  // (and from exactly 128 KiB a CU on: 4096 x 4096 at 96 / 128 rows 19.7 / 22.0 us with the adding kernel, which
+  // also does the add, against 17.2 / 19.3 for the library's product, whose result the norm kernel then adds)
+  if (M > 64) return (epilogue == WEPI_ACCUM && S > 1 && (long)N * K * 2 >= 131072L * cus) ? 1 : 0;
   // from 9 to 16 rows the gated product of a wide feed-forward (up to 8 rows the other kernel, whose
   // workgroups stay and keep two runs a wave in flight, is ahead: 24576 x 4096 36 us against 37, 51200 x
   // 5120 91 to 97 against 101 to 103): one K range, enough workgroups to fill the
