@@ -11,6 +11,9 @@
 // element-type tags of the C interface
 enum { RA_F32 = 0, RA_BF16 = 1 };
 
+// XCDs of the chip: workgroups are dealt round them in the order of their numbers, each XCD has an L2 of its own
+#define RA_XCDS 8
+
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));

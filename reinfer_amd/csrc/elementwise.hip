@@ -410,99 +410,235 @@ qk_norm_rope_cache_head_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w,
   }
 }
 
+// 16 bytes of a row, as floats
+template <typename T> struct Row16;
+template <> struct Row16<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void widen(f32x4_raw v, float* o) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = v[i];
+  }
+  static __device__ __forceinline__ void load(const float* p, float* o) {
+    const f32x4_raw v = *(const f32x4_raw*)p;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = v[i];
+  }
+  static __device__ __forceinline__ void store(float* p, const float* v) {
+    *(f32x4_raw*)p = (f32x4_raw){v[0], v[1], v[2], v[3]};
+  }
+};
+template <> struct Row16<bf16_t> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void widen(f32x4_raw raw, float* o) {
+    const bf16x8_t v = __builtin_bit_cast(bf16x8_t, raw);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (float)v[i];
+  }
+  static __device__ __forceinline__ void load(const bf16_t* p, float* o) {
+    const bf16x8_t v = *(const bf16x8_t*)p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (float)v[i];
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float* v) {
+    bf16x8_t o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (bf16_t)v[i];
+    *(bf16x8_t*)p = o;
+  }
+};
+
 // The same for the common shape (half-split rotation over the whole head, head
 // size a power of two between 16 and 256): one workgroup per token. The sines and
 // cosines of the token's angles are computed once, in LDS, for all heads (the
-// plain kernel computes them per head); a head is spread over d/8 lanes, each
-// holding rotation pairs (j..j+3, j+d/2..j+d/2+3) as two 4-element vectors.
+// plain kernel computes them per head); a head is spread over LPH lanes, each
+// holding 16 bytes of either half of the head: rotation pairs (j..j+E-1, j+d/2..j+d/2+E-1).
+//
+// What it lasts is how its accesses reach memory, not its arithmetic (timed with parts left out at 8192
+// tokens of 48 heads of 128: neither the sines nor the barrier count). With 8 bytes a lane the reads ran at
+// 3.0 TB/s, with 16 at 5. A token's keys and values go into tiles in which the same elements of
+// neighbouring slots lie side by side: written token by token they are pieces of 16 bytes (keys) or single
+// elements (values), each a request of its own. So four tokens in a row whose slots are s .. s + 3 with s a
+// multiple of 4 (the usual case inside a prompt) share the work on their keys and values: workgroup i of
+// the four takes KV heads i, i + 4, ... of all four tokens, lays the rotated keys and the values out in
+// LDS as the tiles want them and writes runs of 64 bytes (keys) and whole 128-byte lines (values).
+// 8192 tokens: 68 -> 55 us with 16-byte accesses and the XCD order below, -> 50 with the shared tiles, -> 46
+// with the query rows asked for before the angles (2048 tokens, one round of workgroups: 15.3 -> 13.5 us).
+// Dynamic LDS: the sines of four tokens (4 * d floats) and the two staging areas (qk_token_lds below).
 template <typename TA, typename TW, int LPH>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_cache_token_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w, const TW* __restrict__ k_w,
                                 float eps, const int* __restrict__ positions,
                                 const float* __restrict__ inv_freq, const int* __restrict__ slots,
                                 TA* __restrict__ kcache, TA* __restrict__ vcache, int block_size, int Hq,
-                                int Hkv, int d) {
-  __shared__ float cs[128], sn[128];
-  const int t = blockIdx.x;
+                                int Hkv, int d, int T, int share) {
+  constexpr int E = Row16<TA>::E;
+  constexpr int ROWS = 256 / LPH;              // head rows a pass of the workgroup
+  extern __shared__ __attribute__((aligned(16))) unsigned char qk_lds[];
   const int half = d / 2;
-  const float pos = (float)positions[t];
-  for (int j = threadIdx.x; j < half; j += blockDim.x) sincosf(pos * inv_freq[j], &sn[j], &cs[j]);
-  __syncthreads();
+  float* cs = (float*)qk_lds;                  // [4][half]
+  float* sn = cs + 4 * half;                   // [4][half]
+  // Sixteen tokens in a row write into the same lines of the cache (a tile's 16 slots lie side by side) and
+  // workgroups go round the chip's XCDs, each with an L2 of its own: a run of 16 tokens is given to one
+  // XCD (workgroup w runs on XCD w % RA_XCDS), so that the pieces meet in one L2. The grid is padded to
+  // runs for all XCDs; a workgroup past the last token has nothing to do.
+  const int w_xcd = blockIdx.x % RA_XCDS, w_k = blockIdx.x / RA_XCDS;
+  const int t = ((w_k / 16) * RA_XCDS + w_xcd) * 16 + w_k % 16;
+  if (t >= T) return;
   const int n_heads = Hq + 2 * Hkv;
   const int sub = threadIdx.x / LPH, ln = threadIdx.x % LPH;
-  const int j0 = ln * 4;                       // pairs j0..j0+3
+  const int j0 = ln * E;                       // pairs j0..j0+E-1
   const int slot = slots[t];
-  const size_t blk = slot >= 0 ? (size_t)(slot / block_size) : 0;
-  const int off = slot >= 0 ? slot % block_size : 0;
-  // In the V tile the same element of four neighbouring slots lies side by side: four tokens in a row whose
-  // slots are s, s + 1, s + 2, s + 3 with s a multiple of 4 (the usual case inside a prompt) have their values
-  // written by the first of the four workgroups, 16 contiguous elements a thread, instead of element by
-  // element by each (2048 tokens, 8 value heads of 128: 16.5 -> 12 us).
-  const int t0 = t & ~3;
-  bool quad = t0 + 3 < (int)gridDim.x;
+  const int t0 = t & ~3, me = t - t0;
+  // the first pass's query rows are asked for before anything they do not hang on is waited for
+  f32x4_raw first_a = {}, first_c = {};
+  if (sub < Hq) {
+    const TA* u = qkv + ((size_t)t * n_heads + sub) * d;
+    first_a = *(const f32x4_raw*)(u + j0);
+    first_c = *(const f32x4_raw*)(u + half + j0);
+  }
+  bool quad = share && t0 + 3 < T;             // the same in every thread of the workgroup
+  int s0 = -1;
   if (quad) {
-    const int s0 = slots[t0];
+    s0 = slots[t0];
     quad = s0 >= 0 && (s0 & 3) == 0 && slots[t0 + 1] == s0 + 1 && slots[t0 + 2] == s0 + 2 && slots[t0 + 3] == s0 + 3;
   }
-  for (int head = sub; head < n_heads; head += 256 / LPH) {
-    TA* u = qkv + ((size_t)t * n_heads + head) * d;
-    const bool is_q = head < Hq;
-    const bool is_k = !is_q && head < Hq + Hkv;
-    const int kvh = is_q ? 0 : (is_k ? head - Hq : head - Hq - Hkv);
-    if (!is_q && slot < 0) continue;           // nothing to store for this token
-    if (!is_q && !is_k && quad) continue;      // written below, four tokens at once
-    f32x4_raw a = Vec4<TA>::load(u + j0), c = Vec4<TA>::load(u + half + j0);
-    TA* slab = (is_q ? nullptr : (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d);
-    if (!is_q && !is_k) {                      // v head: copy into the V tile order
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        slab[cache_v_index(off, j0 + i, d)] = from_f32<TA>(a[i]);
-        slab[cache_v_index(off, half + j0 + i, d)] = from_f32<TA>(c[i]);
-      }
-      continue;
+  if (quad) {
+    for (int idx = threadIdx.x; idx < 4 * half; idx += blockDim.x) {
+      const int tok = idx / half, j = idx % half;
+      sincosf((float)positions[t0 + tok] * inv_freq[j], &sn[idx], &cs[idx]);
     }
-    const TW* w = is_q ? q_w : k_w;
+  } else {
+    const float pos = (float)positions[t];
+    for (int j = threadIdx.x; j < half; j += blockDim.x) sincosf(pos * inv_freq[j], &sn[me * half + j], &cs[me * half + j]);
+  }
+  __syncthreads();
+
+  // one head row: norm and rotation with the angles of token `tok` of the four
+  auto turn_held = [&](f32x4_raw raw_a, f32x4_raw raw_c, const TW* w, int tok, float* ra, float* rc) {
+    float a[E], c[E];
+    Row16<TA>::widen(raw_a, a);
+    Row16<TA>::widen(raw_c, c);
     if (w) {
-      float ss = a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3] + c[0] * c[0] + c[1] * c[1] + c[2] * c[2] + c[3] * c[3];
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < E; ++i) ss += a[i] * a[i];
+#pragma unroll
+      for (int i = 0; i < E; ++i) ss += c[i] * c[i];
 #pragma unroll
       for (int m = LPH / 2; m > 0; m >>= 1) ss += __shfl_xor(ss, m, RA_WAVE);
       const float rstd = rsqrtf(ss / (float)d + eps);
-      a = a * rstd * Vec4<TW>::load(w + j0);
-      c = c * rstd * Vec4<TW>::load(w + half + j0);
-    }
-    f32x4_raw ra, rc;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = a[i] * cs[j0 + i] - c[i] * sn[j0 + i];
-      rc[i] = a[i] * sn[j0 + i] + c[i] * cs[j0 + i];
-    }
-    if (is_q) {
-      Vec4<TA>::store(u + j0, ra);
-      Vec4<TA>::store(u + half + j0, rc);
-    } else {                                   // four elements of one 8-chunk are contiguous in the K tile
-      Vec4<TA>::store(slab + cache_k_index(off, j0, d), ra);
-      Vec4<TA>::store(slab + cache_k_index(off, half + j0, d), rc);
-    }
-  }
-  if (quad && t == t0) {
-    // thread: one value head, elements e0 .. e0 + 3 of the four tokens -> [element][token], 16 in a row
-    const int per_head = d / 4;
-    for (int it = threadIdx.x; it < Hkv * per_head; it += blockDim.x) {
-      const int kvh = it / per_head, e0 = (it % per_head) * 4;
-      TA v[4][4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const TA* src = qkv + ((size_t)(t0 + i) * n_heads + Hq + Hkv + kvh) * d + e0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[i][j] = src[j];
+      for (int i = 0; i < E; ++i) {
+        a[i] = a[i] * rstd * to_f32(w[j0 + i]);
+        c[i] = c[i] * rstd * to_f32(w[half + j0 + i]);
       }
-      TA* dst = vcache + (blk * Hkv + kvh) * (size_t)block_size * d + cache_v_index(off, e0, d);
+    }
+    const float* csr = cs + tok * half + j0;
+    const float* snr = sn + tok * half + j0;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+    for (int i = 0; i < E; ++i) {
+      ra[i] = a[i] * csr[i] - c[i] * snr[i];
+      rc[i] = a[i] * snr[i] + c[i] * csr[i];
+    }
+  };
+  auto turn = [&](const TA* u, const TW* w, int tok, float* ra, float* rc) {
+    turn_held(*(const f32x4_raw*)(u + j0), *(const f32x4_raw*)(u + half + j0), w, tok, ra, rc);
+  };
+
+  // the token's own query heads, in place
+  for (int head = sub; head < Hq; head += ROWS) {
+    TA* u = qkv + ((size_t)t * n_heads + head) * d;
+    float ra[E], rc[E];
+    if (head == sub) turn_held(first_a, first_c, q_w, me, ra, rc);
+    else turn(u, q_w, me, ra, rc);
+    Row16<TA>::store(u + j0, ra);
+    Row16<TA>::store(u + half + j0, rc);
+  }
+
+  if (!quad) {                                 // its own keys and values, piece by piece
+    if (slot < 0) return;                      // nothing to store for this token
+    const size_t blk = (size_t)(slot / block_size);
+    const int off = slot % block_size;
+    for (int r = sub; r < 2 * Hkv; r += ROWS) {
+      const bool is_k = r < Hkv;
+      const int kvh = is_k ? r : r - Hkv;
+      const TA* u = qkv + ((size_t)t * n_heads + Hq + r) * d;
+      TA* slab = (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d;
+      if (is_k) {                              // the elements of one 8-chunk are contiguous in the K tile
+        float ra[E], rc[E];
+        turn(u, k_w, me, ra, rc);
+        Row16<TA>::store(slab + cache_k_index(off, j0, d), ra);
+        Row16<TA>::store(slab + cache_k_index(off, half + j0, d), rc);
+      } else {
+        float a[E], c[E];
+        Row16<TA>::load(u + j0, a);
+        Row16<TA>::load(u + half + j0, c);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[j * 4 + i] = v[i][j];
+        for (int i = 0; i < E; ++i) {
+          slab[cache_v_index(off, j0 + i, d)] = from_f32<TA>(a[i]);
+          slab[cache_v_index(off, half + j0 + i, d)] = from_f32<TA>(c[i]);
+        }
+      }
+    }
+    return;
+  }
+
+  // KV heads me, me + 4, ... of the four tokens: into LDS in tile order, then out in whole runs.
+  //   keys    kst[m][chunk][token][8]      = the K tile's [chunk][slot][8] over the four slots
+  //   values  vst[m][e / 16][e % 16][token] = the V tile's [e / 16][slot / 4][e % 16][slot % 4] of this quad
+  const int n_mine = (Hkv - me + 3) / 4;       // may be 0
+  const int n_max = (Hkv + 3) / 4;
+  TA* kst = (TA*)(sn + 4 * half);
+  TA* vst = kst + (size_t)n_max * d * 4;
+  for (int r = sub; r < n_mine * 8; r += ROWS) {
+    const int m = r >> 3, tok = r & 3;
+    const bool is_k = (r & 4) == 0;
+    const int kvh = me + 4 * m;
+    const TA* u = qkv + ((size_t)(t0 + tok) * n_heads + Hq + (is_k ? 0 : Hkv) + kvh) * d;
+    if (is_k) {
+      float ra[E], rc[E];
+      turn(u, k_w, tok, ra, rc);
+      TA* dst = kst + (size_t)m * d * 4;
+      // element e of the row -> ((e / 8) * 4 + tok) * 8 + e % 8; the E elements of a lane lie in one chunk
+      Row16<TA>::store(dst + ((j0 >> 3) * 4 + tok) * 8 + (j0 & 7), ra);
+      Row16<TA>::store(dst + (((half + j0) >> 3) * 4 + tok) * 8 + ((half + j0) & 7), rc);
+    } else {
+      float a[E], c[E];
+      Row16<TA>::load(u + j0, a);
+      Row16<TA>::load(u + half + j0, c);
+      TA* dst = vst + (size_t)m * d * 4;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        dst[(j0 + i) * 4 + tok] = from_f32<TA>(a[i]);
+        dst[(half + j0 + i) * 4 + tok] = from_f32<TA>(c[i]);
+      }
     }
   }
+  __syncthreads();
+  constexpr int PIECE = 16 / (int)sizeof(TA);  // elements of a 16-byte piece
+  const size_t blk = (size_t)(s0 / block_size);
+  const int off0 = s0 % block_size;            // a multiple of 4: the four slots lie in one tile
+  const size_t tile_at = (size_t)(off0 >> 4) * 16 * d;
+  const int per_head = d * 4 / PIECE;          // pieces of a head's four tokens
+  for (int idx = threadIdx.x; idx < n_mine * per_head * 2; idx += blockDim.x) {
+    const bool is_k = idx < n_mine * per_head;
+    const int i2 = is_k ? idx : idx - n_mine * per_head;
+    const int m = i2 / per_head, e4 = (i2 % per_head) * PIECE;     // element among the head's d * 4
+    const int kvh = me + 4 * m;
+    TA* slab = (is_k ? kcache : vcache) + (blk * Hkv + kvh) * (size_t)block_size * d + tile_at;
+    const TA* src = (is_k ? kst : vst) + (size_t)m * d * 4 + e4;
+    // keys: chunk c = e4 / 32 holds 32 elements of the four tokens, at (c * 16 + off0 % 16) * 8 in the tile;
+    // values: group g = e4 / 64 holds 64, at ((g * 4 + (off0 % 16) / 4) * 16) * 4
+    const size_t at = is_k ? (size_t)((e4 >> 5) * 16 + (off0 & 15)) * 8 + (e4 & 31)
+                           : (size_t)((e4 >> 6) * 4 + ((off0 & 15) >> 2)) * 64 + (e4 & 63);
+    *(f32x4_raw*)(slab + at) = *(const f32x4_raw*)src;
+  }
+}
+
+// Bytes of dynamic LDS of the per-token kernel: the sines and cosines of four tokens and, where four
+// tokens share their keys and values, the two staging areas.
+static size_t qk_token_lds(int Hkv, int d, size_t elem, bool share) {
+  return (size_t)4 * d * sizeof(float) + (share ? (size_t)2 * ((Hkv + 3) / 4) * d * 4 * elem : 0);
 }
 
 static int qk_norm_rope_cache_impl(void* qkv, int act_dtype, const void* q_weight, const void* k_weight,
@@ -527,21 +663,26 @@ static int qk_norm_rope_cache_impl(void* qkv, int act_dtype, const void* q_weigh
   const bool pow2 = (d & (d - 1)) == 0 && d >= 16 && d <= 256;
   if (!sm.parts && pow2 && n_tokens >= 192 && rope_style == 0 && rotary_dim == d && ((uintptr_t)qkv % 16) == 0 &&
       (q_weight == nullptr || (((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0))) {
+    // four tokens share their keys and values where the staging areas leave room for eight workgroups a CU
+    const bool share = qk_token_lds(Hkv, d, act_dtype == RA_F32 ? 4 : 2, true) <= 16384;
 #define RA_TOK2(TA, TW, LPH)                                                                              \
-  qk_norm_rope_cache_token_kernel<TA, TW, LPH><<<n_tokens, 256, 0, stream>>>(                             \
+  qk_norm_rope_cache_token_kernel<TA, TW, LPH>                                                            \
+      <<<(n_tokens + 16 * RA_XCDS - 1) / (16 * RA_XCDS) * (16 * RA_XCDS), 256,                            \
+         qk_token_lds(Hkv, d, sizeof(TA), share), stream>>>(                                              \
       (TA*)qkv, (const TW*)q_weight, (const TW*)k_weight, eps, positions, inv_freq, slots, (TA*)kcache,  \
-      (TA*)vcache, block_size, Hq, Hkv, d)
-#define RA_TOK(TA, TW)                       \
-  do {                                       \
-    if (d == 16) RA_TOK2(TA, TW, 2);         \
-    else if (d == 32) RA_TOK2(TA, TW, 4);    \
-    else if (d == 64) RA_TOK2(TA, TW, 8);    \
-    else if (d == 128) RA_TOK2(TA, TW, 16);  \
-    else RA_TOK2(TA, TW, 32);                \
+      (TA*)vcache, block_size, Hq, Hkv, d, n_tokens, share ? 1 : 0)
+  /* lanes a head: 16 bytes of either half a lane (SH: 0 for 4-byte elements, 1 for 2-byte ones) */
+#define RA_TOK(TA, TW, SH)                           \
+  do {                                               \
+    if (d == 16) RA_TOK2(TA, TW, (2 >> SH));         \
+    else if (d == 32) RA_TOK2(TA, TW, (4 >> SH));    \
+    else if (d == 64) RA_TOK2(TA, TW, (8 >> SH));    \
+    else if (d == 128) RA_TOK2(TA, TW, (16 >> SH));  \
+    else RA_TOK2(TA, TW, (32 >> SH));                \
   } while (0)
-    if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_TOK(float, float);
-    else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_TOK(bf16_t, bf16_t);
-    else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_TOK(bf16_t, float);
+    if (act_dtype == RA_F32 && weight_dtype == RA_F32) RA_TOK(float, float, 0);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_BF16) RA_TOK(bf16_t, bf16_t, 1);
+    else if (act_dtype == RA_BF16 && weight_dtype == RA_F32) RA_TOK(bf16_t, float, 1);
     else return ra_fail("qk_norm_rope_cache: unsupported dtypes (activations %d, weight %d)", act_dtype, weight_dtype);
 #undef RA_TOK
 #undef RA_TOK2

@@ -204,7 +204,8 @@ def test_qk_norm_rope_cache(dtype, Hq, Hkv, d, rot, style, norm, T):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("Hq,Hkv,d", [(4, 2, 16), (5, 5, 128), (32, 8, 128), (2, 1, 256), (6, 3, 64)])
+@pytest.mark.parametrize("Hq,Hkv,d", [(4, 2, 16), (5, 5, 128), (32, 8, 128), (2, 1, 256), (6, 3, 64), (40, 40, 128),
+                                      (9, 9, 32)])
 def test_qk_norm_rope_cache_values_of_four_slots_in_a_row(dtype, Hq, Hkv, d):
     """A prompt's tokens sit in slots that follow each other: where four tokens in a row fill slots 4k .. 4k + 3
     the per-token kernel writes their values in one piece. Runs of slots that start at a multiple of 4, one that
@@ -217,20 +218,31 @@ def test_qk_norm_rope_cache_values_of_four_slots_in_a_row(dtype, Hq, Hkv, d):
     slots_l = [32 + t for t in range(80)] + [321 + t for t in range(40)] + [480 + t for t in range(83)]
     slots_l[50] = -1
     slots = torch.tensor(slots_l, dtype=torch.int32, device=DEV)
-    positions = torch.arange(T, dtype=torch.int32, device=DEV)
+    # every token another position, all below 128: the kernel's angles are floats, whose rounding grows with the position
+    positions = ((torch.arange(T, dtype=torch.int32) * 5) % 128).to(DEV)
     kc = torch.full((nblk, Hkv, bs // 16, 16 * d), float("nan"), device=DEV, dtype=DT[dtype])
     vc = torch.full_like(kc, float("nan"))
     inv_freq = (10000.0 ** (-torch.arange(0, d, 2).double() / d)).float().to(DEV)
-    ops().qk_norm_rope_cache(qkv, None, None, 1e-6, positions, inv_freq, d, 0, slots, kc, vc, Hq, Hkv, d)
-    v = src.view(T, Hq + 2 * Hkv, d)[:, Hq + Hkv:]
-    vc = unpack_v(vc, d)
+    qw = (torch.rand(d, device=DEV) + 0.5).to(DT[dtype])
+    kw = (torch.rand(d, device=DEV) + 0.5).to(DT[dtype])
+    ops().qk_norm_rope_cache(qkv, qw, kw, 1e-6, positions, inv_freq, d, 0, slots, kc, vc, Hq, Hkv, d)
+    u = src.view(T, Hq + 2 * Hkv, d)
+    v = u[:, Hq + Hkv:]
+    # the four tokens of such a group also share the work on their keys, each with the angles of its own position
+    q_ref = plain.rope_neox(plain.head_norm(u[:, :Hq].double().cpu(), qw.double().cpu(), 1e-6), positions.cpu(), 10000.0)
+    k_ref = plain.rope_neox(plain.head_norm(u[:, Hq:Hq + Hkv].double().cpu(), kw.double().cpu(), 1e-6),
+                            positions.cpu(), 10000.0)
+    close(qkv.view(T, -1, d)[:, :Hq], q_ref, OUT_TOL[dtype])
+    vc, kc = unpack_v(vc, d), unpack_k(kc, d)
     written = torch.zeros(nblk, bs, dtype=torch.bool)
     for t, sl in enumerate(slots_l):
         if sl < 0:
             continue
         written[sl // bs, sl % bs] = True
         assert torch.equal(vc[sl // bs, :, sl % bs, :], v[t]), t
+        close(kc[sl // bs, :, sl % bs, :], k_ref[t], OUT_TOL[dtype])
     assert torch.isnan(vc.float().cpu().permute(0, 2, 1, 3)[~written]).all()
+    assert torch.isnan(kc.float().cpu().permute(0, 2, 1, 3)[~written]).all()
 
 
 @pytest.mark.parametrize("Hq,Hkv,d,rot,style,norm", [(4, 2, 16, 16, 0, True), (3, 1, 80, 32, 0, False),
