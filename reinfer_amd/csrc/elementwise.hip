@@ -488,7 +488,9 @@ qk_norm_rope_cache_token_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w
   const int sub = threadIdx.x / LPH, ln = threadIdx.x % LPH;
   const int j0 = ln * E;                       // pairs j0..j0+E-1
   const int slot = slots[t];
-  const int t0 = t & ~3, me = t - t0;
+  // which of four tokens this one is follows from its slot, not from its place in the step: a portion
+  // that begins behind a few single tokens still finds its groups
+  const int me = slot >= 0 ? (slot & 3) : 0, t0 = t - me;
   // the first pass's query rows are asked for before anything they do not hang on is waited for
   f32x4_raw first_a = {}, first_c = {};
   if (sub < Hq) {
@@ -496,12 +498,9 @@ qk_norm_rope_cache_token_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w
     first_a = *(const f32x4_raw*)(u + j0);
     first_c = *(const f32x4_raw*)(u + half + j0);
   }
-  bool quad = share && t0 + 3 < T;             // the same in every thread of the workgroup
-  int s0 = -1;
-  if (quad) {
-    s0 = slots[t0];
-    quad = s0 >= 0 && (s0 & 3) == 0 && slots[t0 + 1] == s0 + 1 && slots[t0 + 2] == s0 + 2 && slots[t0 + 3] == s0 + 3;
-  }
+  bool quad = share && slot >= 0 && t0 >= 0 && t0 + 3 < T;      // the same in every thread of the workgroup
+  const int s0 = slot - me;
+  if (quad) quad = slots[t0] == s0 && slots[t0 + 1] == s0 + 1 && slots[t0 + 2] == s0 + 2 && slots[t0 + 3] == s0 + 3;
   if (quad) {
     for (int idx = threadIdx.x; idx < 4 * half; idx += blockDim.x) {
       const int tok = idx / half, j = idx % half;
