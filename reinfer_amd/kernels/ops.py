@@ -483,6 +483,7 @@ class HipKernels:
     # 1 / 4 / 16 / 64 tokens: 17.9 / 35.9 / 113 / 370 against 14.7 / 31.2 / 101 / 364)
     DECODE_WIDE_PAIRS = 64
     DECODE_WIDE_CTX = 4096      # keys of head size 128: what counts is the bytes of a (token, KV head) pair
+    DECODE_WIDE_FILL = 0.9      # of the last round of large workgroups that the pairs must fill
 
     def _slots_of_decode(self, num_heads: int, num_kv_heads: int, head_dim: int, waves: int) -> int:
         """Workgroups of the decode kernel's form with ``waves`` waves that the chip holds at once (0: that
@@ -513,7 +514,7 @@ class HipKernels:
             wide = self._slots_of_decode(num_heads, num_kv_heads, head_dim, 12)
             # whole rounds of the large workgroups, or nearly (64 requests over 8 KV heads are two rounds
             # of 256: 8.45 ms a step against 8.65 with the small workgroups)
-            if wide > 0 and pairs >= 0.9 * (-(-pairs // wide) * wide):
+            if wide > 0 and pairs >= self.DECODE_WIDE_FILL * (-(-pairs // wide) * wide):
                 waves = 12
         slots = self._slots_of_decode(num_heads, num_kv_heads, head_dim, waves) or 768
         least = 256 if waves == 4 else 512
