@@ -39,6 +39,7 @@ struct WideNorm {
   bf16_t* out_x;           // [M, out_ldx] bf16(C_new * out_w)
   int out_ldx;
   float* out_ss;           // [ceil(N / 1024), M] sums of squares of C_new over 1024 columns
+  float out_eps;           // >= 0 with out_ss null: the adding kernel finishes the norm, out_x = bf16(norm(C_new) * out_w)
 };
 
 #define GW_KS 128                      // k elements of a run
@@ -335,6 +336,71 @@ gemm_wide_reduce_kernel(const float* __restrict__ P, int S, const bf16_t* __rest
   }
 }
 
+// The same with a whole row a workgroup, which then also finishes the RMSNorm that follows an accumulating
+// product: out_x = bf16(C_new * rsqrt(mean(C_new^2) + out_eps) * out_w). For the rows above those that the
+// weight-streaming products take (65 to 128 requests decoding), where the products behind the norm are the
+// library's and cannot apply a row factor: the norm then costs no kernel of its own. 1024 threads a row, each
+// with CH chunks of 4 columns (N <= 4096 CH, N a multiple of 4): with few workgroups it is the loads in flight
+// that count (256 threads with four chunks each, one after the other: 11 us against 7).
+template <int CH>
+__global__ void __launch_bounds__(1024)
+gemm_wide_reduce_rows_kernel(const float* __restrict__ P, int S, const bf16_t* __restrict__ bias,
+                             float* __restrict__ C, int ldc, int M, int N, WideNorm nf) {
+  __shared__ float red[17];
+  const int m = blockIdx.x;
+  float rstd = 1.f;
+  if (nf.in_ss) {                              // the same for every thread: the threads share the parts out
+    float t = 0.f;
+    for (int p = threadIdx.x; p < nf.in_parts; p += blockDim.x) t += nf.in_ss[(size_t)p * M + m];
+    rstd = rsqrtf(block_sum(t, red) * nf.in_inv_width + nf.in_eps);
+  }
+  float x[CH][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int n = (c * 1024 + threadIdx.x) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[c][i] = 0.f;
+    if (n >= N) continue;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    constexpr int U = 6;                       // ranges asked for in one trip, added in range order
+    for (int s0 = 0; s0 < S; s0 += U) {
+      f32x4_t t[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) t[j] = *(const f32x4_t*)(P + ((size_t)min(s0 + j, S - 1) * M + m) * N + n);
+#pragma unroll
+      for (int j = 0; j < U; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += s0 + j < S ? t[j][i] : 0.f;
+    }
+    const f32x4_t c0 = *(const f32x4_t*)(C + (size_t)m * ldc + n);
+    f32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float y = v[i] * rstd;
+      if (bias) y += to_f32(bias[n + i]);
+      y += c0[i];
+      o[i] = y;
+      x[c][i] = y;
+      ss += y * y;
+    }
+    *(f32x4_t*)(C + (size_t)m * ldc + n) = o;
+  }
+  const float rout = rsqrtf(block_sum(ss, red) / (float)N + nf.out_eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int n = (c * 1024 + threadIdx.x) * 4;
+    if (n >= N) continue;
+    bf16x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float w = nf.out_w_f32 ? ((const float*)nf.out_w)[n + i] : to_f32(((const bf16_t*)nf.out_w)[n + i]);
+      o[i] = from_f32<bf16_t>(x[c][i] * rout * w);
+    }
+    *(bf16x4_t*)(nf.out_x + (size_t)m * nf.out_ldx + n) = o;
+  }
+}
+
 // How [M, N, K] is cut: waves a workgroup (5 to 8, 16 features each) and K ranges. With many features
 // one range, and the workgroup width that fills the chip's 256 CUs most evenly (24576 features: 256
 // workgroups of 96; 19456: 244 of 80; 51200: 458 of 112). With few features 128 a workgroup and as many K ranges as
@@ -430,6 +496,13 @@ extern "C" int ra_gemm_wide_row_parts(int N) { return (N + 1023) / 1024; }
 // the second half of a product cut into K ranges: adds them in range order and applies the epilogue
 static int launch_wide_reduce(const void* bias, void* C, int ldc, int out_dtype, int epilogue, int M, int N, int S,
                               const float* scratch, const WideNorm& nf, hipStream_t stream) {
+  if (nf.out_x && !nf.out_ss) {                // a whole row a workgroup: the norm that follows is finished here
+    if (N <= 4096) gemm_wide_reduce_rows_kernel<1><<<M, 1024, 0, stream>>>(scratch, S, (const bf16_t*)bias, (float*)C, ldc, M, N, nf);
+    else if (N <= 8192) gemm_wide_reduce_rows_kernel<2><<<M, 1024, 0, stream>>>(scratch, S, (const bf16_t*)bias, (float*)C, ldc, M, N, nf);
+    else gemm_wide_reduce_rows_kernel<4><<<M, 1024, 0, stream>>>(scratch, S, (const bf16_t*)bias, (float*)C, ldc, M, N, nf);
+    RA_LAUNCH_CHECK("gemm_wide reduce rows");
+    return 0;
+  }
   const dim3 rg((N + 1023) / 1024, M);
 #define RA_GR(EPI, TO) \
   gemm_wide_reduce_kernel<EPI, TO><<<rg, 256, 0, stream>>>(scratch, S, (const bf16_t*)bias, (TO*)C, ldc, M, N, nf)
@@ -490,7 +563,7 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
                                    int epilogue, int M, int N, int K, int lda, int ldc, float* scratch,
                                    long scratch_floats, const float* in_ss, int in_parts, float in_eps,
                                    int in_width, const void* out_w, int out_w_dtype, void* out_x, int out_ldx,
-                                   float* out_ss, hipStream_t stream) {
+                                   float* out_ss, float out_eps, hipStream_t stream) {
   RA_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: empty product (%d, %d, %d)", M, N, K);
   RA_CHECK(M <= 128, "gemm_wide: %d rows; this kernel takes at most 128", M);
   RA_CHECK(K % 8 == 0 && lda % 8 == 0, "gemm_wide: K (%d) and the row stride (%d) must be multiples of 8", K, lda);
@@ -512,9 +585,14 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
     nf.in_inv_width = 1.f / (float)in_width;
   }
   const bool emits = out_x || out_ss || out_w;
+  const bool finishes = emits && !out_ss;      // the adding kernel finishes the norm that follows
   if (emits) {
     RA_CHECK(epilogue == WEPI_ACCUM, "gemm_wide: only the accumulating epilogue emits for a norm");
-    RA_CHECK(out_x && out_ss && out_w, "gemm_wide: emitting needs the norm weight, the scaled copy and the partial sums");
+    RA_CHECK(out_x && out_w && (out_ss || out_eps >= 0.f),
+             "gemm_wide: emitting needs the norm weight, the scaled copy and the partial sums (or, to finish the norm, its eps)");
+    RA_CHECK(!finishes || (N % 4 == 0 && N <= 16384 && ldc % 4 == 0 && out_ldx % 4 == 0 && ((uintptr_t)C % 16) == 0 &&
+                           ((uintptr_t)out_x % 8) == 0),
+             "gemm_wide: finishing the norm takes rows of up to 16384 columns in steps of 4 (%d, strides %d and %d)", N, ldc, out_ldx);
     RA_CHECK(out_w_dtype == RA_BF16 || out_w_dtype == RA_F32, "gemm_wide: unknown norm weight dtype tag %d", out_w_dtype);
     RA_CHECK(out_ldx >= N, "gemm_wide: the scaled copy's row stride (%d) is below %d", out_ldx, N);
     nf.out_w = out_w;
@@ -522,6 +600,7 @@ extern "C" int ra_gemm_wide_normed(const void* A, const void* W, const void* bia
     nf.out_x = (bf16_t*)out_x;
     nf.out_ldx = out_ldx;
     nf.out_ss = out_ss;
+    nf.out_eps = out_eps;
   }
   const long need = ra_gemm_wide_scratch(epilogue, M, N, K, emits);
   RA_CHECK(need == 0 || (scratch && scratch_floats >= need && ((uintptr_t)scratch % 16) == 0),
@@ -587,5 +666,5 @@ extern "C" int ra_gemm_wide(const void* A, const void* W, const void* bias, void
                             int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                             hipStream_t stream) {
   return ra_gemm_wide_normed(A, W, bias, C, out_dtype, epilogue, M, N, K, lda, ldc, scratch, scratch_floats,
-                             nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, stream);
+                             nullptr, 0, 0.f, 0, nullptr, 0, nullptr, 0, nullptr, -1.f, stream);
 }

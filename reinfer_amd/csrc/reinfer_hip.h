@@ -78,12 +78,15 @@ int ra_gemm_wide(const void* A, const void* W, const void* bias, void* C, int ou
                  int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                  hipStream_t stream);
 // With a carried RMSNorm, as ra_gemm_skinny_normed; an emitting product always needs scratch
-// (ra_gemm_wide_scratch with emits = 1) and writes out_ss[ra_gemm_wide_row_parts(N), M].
+// (ra_gemm_wide_scratch with emits = 1) and writes out_ss[ra_gemm_wide_row_parts(N), M]. With out_ss null and
+// out_eps >= 0 it finishes the norm that follows instead: out_x = bf16(norm(C_new, out_eps) * out_w), one
+// workgroup a row (N a multiple of 4, at most 16384).
 int ra_gemm_wide_row_parts(int N);
 int ra_gemm_wide_normed(const void* A, const void* W, const void* bias, void* C, int out_dtype, int epilogue,
                         int M, int N, int K, int lda, int ldc, float* scratch, long scratch_floats,
                         const float* in_ss, int in_parts, float in_eps, int in_width, const void* out_w,
-                        int out_w_dtype, void* out_x, int out_ldx, float* out_ss, hipStream_t stream);
+                        int out_w_dtype, void* out_x, int out_ldx, float* out_ss, float out_eps,
+                        hipStream_t stream);
 
 // The cache of a layer: K and V are [blocks][Hkv][block_size * d], every (block, KV head) slab
 // in tiles of 16 slots laid out in MFMA operand order (cache_k_index, cache_v_index in common.h);

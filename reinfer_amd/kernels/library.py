@@ -41,7 +41,7 @@ _SIGNATURES = {
     "ra_attention_prefill_split": [P, I, P, I, P, P, P, I, P, I, P, P, I, P, P, I, I, I, I, F, I, P],
     "ra_gemm_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_gemm_wide": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P],
-    "ra_gemm_wide_normed": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P, I, F, I, P, I, P, I, P, P],
+    "ra_gemm_wide_normed": [P, P, P, P, I, I, I, I, I, I, I, P, c_long, P, I, F, I, P, I, P, I, P, F, P],
     "ra_gemm_skinny_normed": [P, P, P, P, I, I, I, I, I, I, I, P, I, F, I, P, I, P, I, P, P],
     "ra_gemm_plain": [P, P, P, P, I, I, I, I, I, I, I, P],
     "ra_sample": [P, I, I, I, P, P, P, P, P, P, P],

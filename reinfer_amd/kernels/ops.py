@@ -636,7 +636,7 @@ class HipKernels:
                      out.stride(0), _stream())
 
     def linear_skinny(self, x, weight, out, bias=None, accumulate: bool = False, row_sums=None,
-                      emit=None, wide: Optional[bool] = None) -> None:
+                      emit=None, wide: Optional[bool] = None, finish=None):
         """The weight-streaming product; with ``accumulate`` the float32 ``out`` is added to (with more rows
         than the weight-streaming kernels take, by the library's product).
 
@@ -645,12 +645,34 @@ class HipKernels:
         rsqrt(sum_p ss[p, m] / width + eps); ``emit`` = (w [N], x_out bfloat16 [M, N],
         ss_out float32 [at least skinny_row_parts(M, N), M]), with ``accumulate`` only, also writes
         bf16(out * w) and each workgroup's sums of squares of its columns of ``out``: into the first
-        rows of ss_out, as many as the kernel that ran has workgroups a row; that number comes back."""
+        rows of ss_out, as many as the kernel that ran has workgroups a row; that number comes back.
+        ``finish`` = (w [N], x_out bfloat16 [M, N], eps), with ``accumulate`` and 65 to 128 rows, asks for the
+        finished norm of the new ``out`` instead, x_out = bf16(rmsnorm(out, eps) * w): True comes back where
+        the product that ran wrote it (``can_finish_norm``), False where it only added."""
         M, N, K = self._check_linear(x, weight, out, bias)
         if x.dtype != torch.bfloat16:
             raise TypeError("linear_skinny: bfloat16 only")
         if accumulate and out.dtype != torch.float32:
             raise TypeError("linear_skinny: accumulation is into a float32 matrix")
+        if finish is not None:
+            if not accumulate or row_sums is not None or emit is not None:
+                raise ValueError("linear_skinny: a finished norm rides on a plain accumulating product only")
+            if self.can_finish_norm(M, N, K):
+                w, xo, eps = finish
+                _dev(w, xo)
+                if w.shape != (N,) or not w.is_contiguous() or xo.dtype != torch.bfloat16 or xo.shape != (M, N) \
+                        or xo.stride(1) != 1:
+                    raise ValueError(f"linear_skinny: norm weight {tuple(w.shape)}, finished rows {tuple(xo.shape)} "
+                                     f"{xo.dtype}; expected [{N}] and bfloat16 [{M}, {N}]")
+                need = int(library.load().ra_gemm_wide_scratch(2, M, N, K, 1))
+                scratch = torch.empty(need, dtype=torch.float32, device=x.device)
+                library.call("ra_gemm_wide_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
+                             _tag(out, "linear output"), 2, M, N, K, x.stride(0), out.stride(0), scratch.data_ptr(),
+                             need, None, 0, 0.0, 0, w.data_ptr(), _tag(w, "norm weight"), xo.data_ptr(),
+                             xo.stride(0), None, float(eps), _stream())
+                return True
+            self.linear_skinny(x, weight, out, bias, accumulate=True, wide=wide)
+            return False
         if accumulate and M > 64 and bias is None and row_sums is None and emit is None and wide is None \
                 and not bool(library.load().ra_gemm_wide_preferred(2, M, N, K)):
             # more rows than the weight-streaming kernels take: the library's product, adding in place
@@ -667,6 +689,17 @@ class HipKernels:
     # registers to spare (the first, at 32 and 64 rows, got slower than with a norm kernel).
     NORM_ON_PRODUCTS_ROWS = 64
     NORM_SKINNY_ROWS = 16
+    # Rows up to which the adding kernel of a product cut into K ranges can finish the norm that follows
+    # (a whole row a workgroup): the decode steps above the weight-streaming products' rows, whose other
+    # products are the library's and can apply no row factor.
+    NORM_FINISHED_ROWS = 128
+
+    def can_finish_norm(self, M: int, N: int, K: int) -> bool:
+        """True where ``linear_skinny(..., accumulate=True, finish=)`` writes the finished norm: the rows
+        between the two limits, a product that the kernel with K ranges takes at these rows, rows of up to
+        16384 columns in steps of 8."""
+        return self.NORM_ON_PRODUCTS_ROWS < M <= self.NORM_FINISHED_ROWS and N % 8 == 0 and N <= 16384 \
+            and K % 8 == 0 and bool(library.load().ra_gemm_wide_preferred(2, M, N, K))
 
     def _few_rows(self, what, x, weight, bias, out, epilogue, M, N, K, wide: Optional[bool] = None) -> None:
         """The weight-streaming product for up to 64 rows, by one of two kernels: the one whose
@@ -745,7 +778,7 @@ class HipKernels:
         scratch = torch.empty(need, dtype=torch.float32, device=x.device) if need else None
         library.call("ra_gemm_wide_normed", x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(),
                      _tag(out, "linear output"), epilogue, M, N, K, x.stride(0), out.stride(0), _ptr(scratch),
-                     need, *norm_args, _stream())
+                     need, *norm_args, -1.0, _stream())
         return parts_out
 
     def can_accumulate(self, x: torch.Tensor, weight: torch.Tensor) -> bool:

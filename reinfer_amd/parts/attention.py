@@ -111,6 +111,9 @@ class GroupedQueryAttention:
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(attn, self.w_o):
             # x += attn . Wo^T in the epilogue, which can also prepare the norm that follows
+            if emit is not None and emit.finished:
+                done = ops.linear_skinny(attn, self.w_o, resid, accumulate=True, finish=emit.finish)
+                return emit if done else None
             if emit is not None:
                 written = ops.linear_skinny(attn, self.w_o, resid, accumulate=True, emit=emit.emit)
                 emit.ss = emit.ss[:written]          # as many partial sums a row as the kernel that ran has workgroups

@@ -86,14 +86,23 @@ class NormTarget:
     """Buffers that a part's last product fills for the norm that follows it, when it adds its
     result into the stream itself: ``x`` = bfloat16(new stream * norm.weight), ``ss`` = partial
     sums of squares of the new stream's rows. A part that declares ``emits_for_norm = True``
-    may be given one (``emit=``); it returns it if it filled it."""
+    may be given one (``emit=``); it returns it if it filled it.
+
+    ``finished``: with more rows than a product behind the norm could scale (they are the library's), the
+    part is asked for the whole norm instead, ``x`` = bfloat16(norm(new stream) * norm.weight), and there are
+    no sums; it returns the target only if its product could do that."""
     norm: object
     x: torch.Tensor
-    ss: torch.Tensor
+    ss: Optional[torch.Tensor]
+    finished: bool = False
 
     @property
     def emit(self):
         return self.norm.weight, self.x, self.ss
+
+    @property
+    def finish(self):
+        return self.norm.weight, self.x, self.norm.eps
 
 
 def split_input(x):

@@ -58,9 +58,9 @@ class PreNormBlock:
     def entry_target(self, resid: torch.Tensor):
         """A NormTarget for this block's first norm, for the part that runs before the block, or
         None if the norm or the mixer behind it cannot use one."""
-        if not getattr(self.mixer, "takes_row_scaled", False) or not hasattr(self.mixer_norm, "emit_target"):
+        if not hasattr(self.mixer_norm, "emit_target"):
             return None
-        return self.mixer_norm.emit_target(resid)
+        return self.mixer_norm.emit_target(resid, getattr(self.mixer, "takes_row_scaled", False))
 
     def forward(self, resid: torch.Tensor, delta, batch, cache: Optional[LayerCache], emit=None):
         # A part that declares ``adds_in_place`` also gets the residual stream: where its last
@@ -88,15 +88,14 @@ class PreNormBlock:
 
     @staticmethod
     def _norm(norm, resid, delta, consumer):
-        if getattr(consumer, "takes_row_scaled", False) and hasattr(norm, "emit_target"):
-            return norm.add_norm(resid, delta, scaled_ok=True)
+        if hasattr(norm, "emit_target"):
+            return norm.add_norm(resid, delta, scaled_ok=getattr(consumer, "takes_row_scaled", False))
         if not isinstance(delta, torch.Tensor) and delta is not None:
             delta = None               # a filled target: the sum is already in the stream
         return norm.add_norm(resid, delta)
 
     @staticmethod
     def _target(norm, resid, producer, consumer):
-        if not (getattr(producer, "emits_for_norm", False) and getattr(consumer, "takes_row_scaled", False)
-                and hasattr(norm, "emit_target")):
+        if not (getattr(producer, "emits_for_norm", False) and hasattr(norm, "emit_target")):
             return None
-        return norm.emit_target(resid)
+        return norm.emit_target(resid, getattr(consumer, "takes_row_scaled", False))

@@ -70,6 +70,9 @@ class SwiGLU:
         can_add = getattr(ops, "can_accumulate", None)
         if resid is not None and can_add and can_add(act, self.w_down):
             # x += act . Wd^T in the epilogue, which can also prepare the norm that follows
+            if emit is not None and emit.finished:
+                done = ops.linear_skinny(act, self.w_down, resid, accumulate=True, finish=emit.finish)
+                return emit if done else None
             if emit is not None:
                 written = ops.linear_skinny(act, self.w_down, resid, accumulate=True, emit=emit.emit)
                 emit.ss = emit.ss[:written]          # as many partial sums a row as the kernel that ran has workgroups

@@ -40,24 +40,34 @@ class RMSNorm:
         (``scaled_ok``) there is nothing left to launch.
         """
         if isinstance(delta, NormTarget):
-            if delta.norm is self and scaled_ok and rows is None:
-                return RowScaled(delta.x, delta.ss, self.eps, self.size)
+            if delta.norm is self and rows is None:
+                if delta.finished:
+                    return delta.x             # the product before wrote the finished rows
+                if scaled_ok:
+                    return RowScaled(delta.x, delta.ss, self.eps, self.size)
             delta = None
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=resid.device)
         kernels.current().add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
 
-    def emit_target(self, resid: torch.Tensor) -> Optional[NormTarget]:
+    def emit_target(self, resid: torch.Tensor, consumer_scales: bool = True) -> Optional[NormTarget]:
         """Buffers for a part that adds into ``resid`` with a product that can also prepare this
-        norm (bfloat16, few rows); None where that does not apply."""
+        norm (bfloat16, few rows); None where that does not apply. Up to the rows of the weight-streaming
+        products, and where the part behind the norm applies a row factor (``consumer_scales``), the half-done
+        form; for the rows above them that the adding kernel can still finish, the finished form."""
         ops = kernels.current()
         parts = getattr(ops, "skinny_row_parts", None)
         T = resid.shape[0]
         # the product behind this norm reads rows of this width as 16-byte pieces: a width that is no
         # multiple of 8 goes through the norm kernel and the plain product
-        if parts is None or self.dtype != torch.bfloat16 or T > getattr(ops, "NORM_ON_PRODUCTS_ROWS", 0) \
-                or resid.shape[1] != self.size or self.size % 8 != 0:
+        if parts is None or self.dtype != torch.bfloat16 or resid.shape[1] != self.size or self.size % 8 != 0:
+            return None
+        few = getattr(ops, "NORM_ON_PRODUCTS_ROWS", 0)
+        if few < T <= getattr(ops, "NORM_FINISHED_ROWS", 0):
+            return NormTarget(self, torch.empty((T, self.size), dtype=torch.bfloat16, device=resid.device), None,
+                              finished=True)
+        if T > few or not consumer_scales:
             return None
         return NormTarget(self,
                           torch.empty((T, self.size), dtype=torch.bfloat16, device=resid.device),

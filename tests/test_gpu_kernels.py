@@ -762,6 +762,39 @@ def test_accumulating_product_over_k_ranges_above_64_rows(M):
     close(stream, want + x[:, :1024].double() @ small.double().T, 2 ** -8)
 
 
+@pytest.mark.parametrize("M", [65, 100, 128])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (2048, 12288), (5120, 8192), (8200, 2560)])
+def test_accumulating_product_finishes_the_norm_that_follows(M, N, K):
+    """65 to 128 rows: the kernel that adds the K ranges into the stream holds a whole row a workgroup and
+    writes the RMSNorm of the new row as well (one, two and four chunks of columns a thread; a width that is
+    no multiple of 1024). A product it does not take adds only and says so."""
+    torch.manual_seed(M + N)
+    eps = 1e-5
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    g = (torch.rand(N, device=DEV) + 0.5).to(torch.bfloat16)
+    stream = torch.randn(M, N, device=DEV)
+    new = stream.double() + x.double() @ w.double().T
+    want = new * torch.rsqrt((new * new).mean(dim=1, keepdim=True) + eps) * g.double()
+    assert ops().can_finish_norm(M, N, K)
+    normed = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    assert ops().linear_skinny(x, w, stream, accumulate=True, finish=(g, normed, eps)) is True
+    close(stream, new, 2 ** -8)
+    close(normed, want, OUT_TOL["bfloat16"])
+    # the same rows through the norm kernel
+    ref = torch.empty_like(normed)
+    ops().add_rmsnorm(stream, None, g, eps, ref)
+    close(normed, ref.double(), OUT_TOL["bfloat16"])
+    # a small product goes to the library: added, not normed
+    small = (torch.randn(512, 1024, device=DEV) / 32).to(torch.bfloat16)
+    assert not ops().can_finish_norm(M, 512, 1024) and not ops().can_finish_norm(64, N, K) and not ops().can_finish_norm(129, N, K)
+    s2 = torch.randn(M, 512, device=DEV)
+    want2 = s2.double() + x[:, :1024].double() @ small.double().T
+    n2 = torch.empty(M, 512, device=DEV, dtype=torch.bfloat16)
+    assert ops().linear_skinny(x[:, :1024], small, s2, accumulate=True, finish=(g[:512].contiguous(), n2, eps)) is False
+    close(s2, want2, 2 ** -8)
+
+
 @pytest.mark.parametrize("M,N,K", [(129, 520, 264), (700, 96, 1000), (2048, 1024, 4096), (3072, 80, 176)])
 def test_accumulating_product_of_many_rows_adds_in_the_library(M, N, K):
     """More rows than the weight-streaming kernels take: the library's product reads and writes the float
