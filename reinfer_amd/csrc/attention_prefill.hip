@@ -351,15 +351,14 @@ flash_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restr
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[j][ot][i] *= corr;
           probabilities();
+          big = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) big += p[e];
         }
-        float psum = 0.f;
         bf16x8_t pb;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          psum += p[e];                                  // the same sum as above where nothing was rescaled
-          pb[e] = from_f32<bf16_t>(p[e]);
-        }
-        l[j] += psum;
+        for (int e = 0; e < 8; ++e) pb[e] = from_f32<bf16_t>(p[e]);
+        l[j] += big;                                     // the lane's sum, of the second set where one was computed
         // O^T[d][column] += V^T[d][key] P[key][column], 32 keys per instruction:
         // k-slots (g, e): e < 4 -> key 4g + e of the first 16-key tile, e >= 4 -> of the second
 #pragma unroll
