@@ -246,3 +246,42 @@ def test_a_token_that_ends_a_request_is_read_one_step_late(tmp_path):
     assert eng.runner.graphs is not None and eng.runner.graphs.replays >= 10
     assert eng.cache_stats()["blocks_free"] == eng.cache_stats()["blocks_total"]
     assert not eng.has_unfinished()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [2, 37, 56])
+def test_steps_launched_one_ahead_give_what_steps_resolved_at_once_give(tmp_path, seed):
+    """Random requests (lengths, temperatures, seeds, stop ids, caps, top-k) under random limits (blocks, running
+    requests, step budget, admission; seeds 37 and 56 preempt): once as the engine runs them, decode steps
+    launched before the tokens of the step before are read, once with every step resolved before the next
+    is planned. The same tokens and the same reasons for ending, and every block back."""
+    import random
+    rng = random.Random(seed)
+    which = rng.choice("ABC")
+    dtype = rng.choice(["bfloat16", "float32"])
+    folder = make_folder(tmp_path, which, dtype)
+    raw, _ = read_folder(folder)
+    V = raw["vocab_size"]
+    n = rng.randrange(4, 40)
+    prompts = [random_tokens(rng.randrange(2, 90), V, 1000 * seed + i) for i in range(n)]
+    params = []
+    for i in range(n):
+        stops = tuple(rng.randrange(V) for _ in range(rng.choice([0, 0, 3, 40])))
+        params.append(SamplingParams(temperature=rng.choice([0.0, 0.0, 0.7, 1.3]), seed=rng.randrange(1 << 30),
+                                     max_tokens=rng.randrange(1, 60), stop_token_ids=stops,
+                                     top_k=rng.choice([None, None, 5]), ignore_eos=rng.random() < 0.5))
+    kw = dict(num_blocks=rng.choice([24, 40, 200]), max_num_seqs=rng.choice([4, 16, 64]),
+              max_num_batched_tokens=rng.choice([32, 64, 256]), admission=rng.choice(["peak", "blocks"]))
+    outs = {}
+    for mode in ("ahead", "at once"):
+        eng = engine_for(folder, "cuda:0", dtype=dtype, **kw)
+        if mode == "at once":
+            eng.runner.can_chain = lambda rows: False
+        res = eng.generate(prompts, params)
+        outs[mode] = [(o.token_ids, o.finish_reason) for o in res]
+        stats = eng.cache_stats()
+        assert stats["blocks_free"] == stats["blocks_total"]
+        if mode == "ahead":
+            assert eng.runner.graphs is not None and eng.runner.graphs.replays > 0
+    assert outs["ahead"] == outs["at once"]
+    assert {r for _, r in outs["ahead"]} >= {"length"}
