@@ -338,7 +338,7 @@ qk_norm_rope_cache_head_kernel(TA* __restrict__ qkv, const TW* __restrict__ q_w,
                                float eps, const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                const int* __restrict__ slots, TA* __restrict__ kcache, TA* __restrict__ vcache,
                                int block_size, int Hq, int Hkv) {
-  constexpr int d = 64 * EPL, half = d / 2;
+  constexpr int d = 64 * EPL;
   constexpr int NF = EPL >= 2 ? EPL / 2 : 1;
   const int lane = threadIdx.x & (RA_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / RA_WAVE);      // the same in every lane
