@@ -101,7 +101,6 @@ flash_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restri
     const int n_chunks = cut.n;
     if (ci >= n_chunks) continue;
     const int* table = block_tables + (size_t)seq * max_blocks;
-    const int Hq = Hkv * G;
 
     // second operand of the score product: column r is query head r of the group
     bf16x8_t qreg[NDT];

@@ -80,9 +80,7 @@ mfma_loop_kernel(int iters, float* __restrict__ sink) {
 extern "C" int ra_stream_read(const void* src, long bytes, void* sink, hipStream_t stream) {
   RA_CHECK(src && sink && bytes >= 16 && bytes % 16 == 0 && ((uintptr_t)src % 16) == 0,
            "stream_read: a 16-byte aligned buffer of a multiple of 16 bytes, got %ld", bytes);
-  int dev = 0, cus = 0;
-  hipGetDevice(&dev);
-  hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const int cus = ra_cu_count();
   RA_CHECK(cus > 0, "stream_read: no compute units reported");
   stream_read_kernel<<<cus * 8, 256, 0, stream>>>((const uint4*)src, (size_t)bytes / 16, (unsigned*)sink);
   RA_LAUNCH_CHECK("stream_read");
@@ -97,9 +95,7 @@ extern "C" int ra_mfma_loop(int shape, int iters, int waves_per_cu, void* sink, 
   const bool big = shape == 32;
   RA_CHECK(iters > 0 && waves_per_cu >= 4 && waves_per_cu % 4 == 0 && waves_per_cu <= 32 && sink && flops,
            "mfma_loop: iterations (%d) and waves a CU (%d: a multiple of 4 up to 32)", iters, waves_per_cu);
-  int dev = 0, cus = 0;
-  hipGetDevice(&dev);
-  hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const int cus = ra_cu_count();
   RA_CHECK(cus > 0, "mfma_loop: no compute units reported");
   const int blocks = cus * (waves_per_cu / 4);
   if (big) mfma_loop32_kernel<<<blocks, 256, 0, stream>>>(iters, (float*)sink);
