@@ -484,6 +484,12 @@ class HipKernels:
     DECODE_WIDE_PAIRS = 64
     DECODE_WIDE_CTX = 4096      # keys of head size 128: what counts is the bytes of a (token, KV head) pair
     DECODE_WIDE_FILL = 0.9      # of the last round of large workgroups that the pairs must fill
+    # Fewer pairs than the chip holds large workgroups: one large workgroup a pair, nothing to merge, from this
+    # share of them on (20 to 28 requests over 8 KV heads, 1000 to 7000 keys: 8 to 14 % faster than the small
+    # workgroups with their chunks and merge, 16 requests: equal), and at any number over contexts up to
+    # DECODE_SHORT_CTX keys of head size 128 (600 keys, 1 to 24 requests: 7.8 to 15.2 us against 9.3 to 20.6)
+    DECODE_WIDE_FILL_ONE = 0.6
+    DECODE_SHORT_CTX = 768
 
     def _slots_of_decode(self, num_heads: int, num_kv_heads: int, head_dim: int, waves: int) -> int:
         """Workgroups of the decode kernel's form with ``waves`` waves that the chip holds at once (0: that
@@ -510,8 +516,11 @@ class HipKernels:
         a CU)."""
         pairs = max(1, n_tokens * num_kv_heads)
         waves = 4
+        wide = self._slots_of_decode(num_heads, num_kv_heads, head_dim, 12)
+        if 0 < pairs <= wide and (pairs >= self.DECODE_WIDE_FILL_ONE * wide
+                                  or max_ctx * head_dim <= self.DECODE_SHORT_CTX * 128):
+            return 512, 1, 12
         if pairs >= self.DECODE_WIDE_PAIRS or max_ctx * head_dim > self.DECODE_WIDE_CTX * 128:
-            wide = self._slots_of_decode(num_heads, num_kv_heads, head_dim, 12)
             # whole rounds of the large workgroups, or nearly (64 requests over 8 KV heads are two rounds
             # of 256: 8.45 ms a step against 8.65 with the small workgroups)
             if wide > 0 and pairs >= self.DECODE_WIDE_FILL * (-(-pairs // wide) * wide):
